@@ -1,0 +1,119 @@
+// common.hpp -- shared declarations of libcwick_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/cwick_hip.h"
+
+namespace cwick {
+
+// ---- error reporting -------------------------------------------------------
+// Every extern "C" entry point returns 0 ("declined") after recording why.
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+bool hip_ok(hipError_t e, const char *what);   // records the error text on failure
+
+#define CWICK_REQUIRE(cond, ...)            \
+    do {                                    \
+        if (!(cond)) {                      \
+            ::cwick::set_error(__VA_ARGS__); \
+            return 0;                       \
+        }                                   \
+    } while (0)
+
+#define CWICK_HIP_CALL(expr)                          \
+    do {                                              \
+        if (!::cwick::hip_ok((expr), #expr)) return 0; \
+    } while (0)
+
+// ---- runtime ---------------------------------------------------------------
+bool backend_ready();                       // device 0 is up and selected
+int num_cus();
+// Grow-only scratch keyed by stream.  Valid until the next call on that stream
+// asks for more bytes; kernels enqueued earlier on the stream have finished
+// with it by the time a later enqueue on the same stream touches it.
+void *workspace(hipStream_t s, size_t bytes);
+// A second, independent scratch area on the same stream (staging of host
+// operands by the host-pointer entry points).
+void *staging(hipStream_t s, size_t bytes);
+
+// ---- kernel launchers (one per .hip file) ----------------------------------
+int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
+                      int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
+                      hipStream_t s);
+int launch_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
+                       int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
+                       float scale, float *out, hipStream_t s);
+int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
+                      int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
+                      const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+                       const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                          int64_t kscale_bstride, int batch, int64_t n_keys,
+                          const uint16_t *q_idx, const float *w, int n_idx_heads,
+                          float *scores, hipStream_t s);
+int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
+                hipStream_t s);
+int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,
+                        hipStream_t s);
+int launch_quant_ikeys(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,
+                       hipStream_t s);
+int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s);
+int launch_e4m3_table(float *out256_dev, hipStream_t s);
+
+// ---- device helpers ---------------------------------------------------------
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+// low / high half of a dword holding two bf16
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) {
+    return __builtin_bit_cast(float, w << 16);
+}
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
+    return __builtin_bit_cast(float, w & 0xFFFF0000u);
+}
+// round-to-nearest-even fp32 -> bf16 (finite inputs)
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
+    return f32_to_bf16_rne(lo) | (f32_to_bf16_rne(hi) << 16);
+}
+// Two E4M3 bytes (low or high 16 bits of w) -> two fp32, hardware conversion
+// (OCP E4M3fn on gfx950).
+template <bool HI>
+__device__ __forceinline__ f32x2 e4m3x2_to_f32(uint32_t w) {
+    return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HI);
+}
+// Two E4M3 bytes -> one dword of two bf16.  Every E4M3 value is exactly
+// representable in bf16, so the conversion is exact.
+template <bool HI>
+__device__ __forceinline__ uint32_t e4m3x2_to_bf16x2(uint32_t w) {
+    bf16x2 r = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, 1.0f, HI);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+}  // namespace cwick

@@ -1,0 +1,260 @@
+// gqa_decode.hip -- split-K flash-decoding for one query position over a bf16
+// K/V cache (the decode branch of the reference's mixer_attn,
+// src/q35_model.c:1656-1701: dec_scores / dec_softmax / dec_out_slices).
+//
+// HBM-bound: every K and V row is read exactly once.
+//
+//   grid  = (n_splits, n_kv_heads), 256 threads (4 waves)
+//   A workgroup owns one kv head and one contiguous slice of keys and serves
+//   the `group` query heads that share the kv head (the reference walks cache
+//   rows for the same reason: one row serves every head of its group,
+//   src/q35_model.c:1417-1423).
+//   A key row of head_dim bf16 is read by LPK = head_dim/8 lanes, 16 bytes
+//   (8 dims) per lane, so a wave covers 64/LPK consecutive rows with full
+//   1 KiB coalesced loads.  Each lane keeps `group` partial dots, an xor
+//   butterfly over the LPK lanes leaves the full score in every lane of the
+//   row, so the weight exp(s - m) is available where the V row lands without a
+//   broadcast.  Online softmax per lane group, KB rows per step to amortise
+//   the rescale; the lane groups of a workgroup are merged through LDS, then
+//   (m, l, acc) goes to the workspace and a second kernel merges the splits.
+#include "common.hpp"
+
+namespace cwick {
+
+constexpr int GQA_DEC_THREADS = 256;
+constexpr int GQA_DEC_KB = 4;      // key rows per lane group per step
+
+template <int HD, int GROUP>
+__global__ void __launch_bounds__(GQA_DEC_THREADS)
+gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+                        const uint16_t *__restrict__ Q, int64_t n_keys, int n_kv_heads,
+                        int keys_per_split, float scale,
+                        float *__restrict__ part_acc,   // [n_splits][n_heads][HD]
+                        float *__restrict__ part_ml) {  // [n_splits][n_heads][2]
+    constexpr int LPK = HD / 8;                 // lanes per key row
+    constexpr int NGRP = GQA_DEC_THREADS / LPK; // lane groups per workgroup
+    const int g = blockIdx.y;
+    const int split = blockIdx.x;
+    const int n_heads = n_kv_heads * GROUP;
+    const int tid = threadIdx.x;
+    const int sub = tid % LPK;                  // which 8 dims of the row
+    const int grp = tid / LPK;                  // which lane group
+    const int64_t k_begin = (int64_t)split * keys_per_split;
+    const int64_t k_end = (k_begin + keys_per_split < n_keys) ? k_begin + keys_per_split : n_keys;
+    const int64_t row_stride = (int64_t)n_kv_heads * HD;
+
+    // this lane's 8 query dims for each head of the group, pre-scaled
+    float q[GROUP][8];
+#pragma unroll
+    for (int j = 0; j < GROUP; j++) {
+        const u32x4 w = *(const u32x4 *)(Q + ((size_t)(g * GROUP + j) * HD + sub * 8));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            q[j][2 * i] = bf16lo_to_f32(w[i]) * scale;
+            q[j][2 * i + 1] = bf16hi_to_f32(w[i]) * scale;
+        }
+    }
+
+    float m[GROUP], l[GROUP], acc[GROUP][8];
+#pragma unroll
+    for (int j = 0; j < GROUP; j++) {
+        m[j] = -INFINITY;
+        l[j] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
+    }
+
+    const uint16_t *Kg = K + (size_t)g * HD + sub * 8;
+    const uint16_t *Vg = V + (size_t)g * HD + sub * 8;
+
+    for (int64_t base = k_begin + (int64_t)grp * GQA_DEC_KB; base < k_end;
+         base += (int64_t)NGRP * GQA_DEC_KB) {
+        u32x4 kw[GQA_DEC_KB], vw[GQA_DEC_KB];
+#pragma unroll
+        for (int r = 0; r < GQA_DEC_KB; r++) {
+            // rows past the slice are clamped (their weight is forced to zero below)
+            int64_t t = base + r < k_end ? base + r : k_end - 1;
+            kw[r] = *(const u32x4 *)(Kg + t * row_stride);
+            vw[r] = *(const u32x4 *)(Vg + t * row_stride);
+        }
+        float s[GQA_DEC_KB][GROUP];
+#pragma unroll
+        for (int r = 0; r < GQA_DEC_KB; r++) {
+            float kf[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                kf[2 * i] = bf16lo_to_f32(kw[r][i]);
+                kf[2 * i + 1] = bf16hi_to_f32(kw[r][i]);
+            }
+#pragma unroll
+            for (int j = 0; j < GROUP; j++) {
+                float d = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) d = __builtin_fmaf(q[j][i], kf[i], d);
+                s[r][j] = d;
+            }
+        }
+        // butterfly over the LPK lanes of the row: every lane ends with the full dot
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1)
+#pragma unroll
+            for (int r = 0; r < GQA_DEC_KB; r++)
+#pragma unroll
+                for (int j = 0; j < GROUP; j++) s[r][j] += __shfl_xor(s[r][j], o, 64);
+#pragma unroll
+        for (int r = 0; r < GQA_DEC_KB; r++)
+            if (base + r >= k_end)
+#pragma unroll
+                for (int j = 0; j < GROUP; j++) s[r][j] = -INFINITY;
+
+#pragma unroll
+        for (int j = 0; j < GROUP; j++) {
+            float mx = m[j];
+#pragma unroll
+            for (int r = 0; r < GQA_DEC_KB; r++) mx = fmaxf(mx, s[r][j]);
+            // mx is finite: row `base` itself is always inside the slice
+            const float corr = __expf(m[j] - mx);
+            m[j] = mx;
+            l[j] *= corr;
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[j][i] *= corr;
+#pragma unroll
+            for (int r = 0; r < GQA_DEC_KB; r++) {
+                const float p = __expf(s[r][j] - mx);
+                l[j] += p;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    acc[j][2 * i] = __builtin_fmaf(p, bf16lo_to_f32(vw[r][i]), acc[j][2 * i]);
+                    acc[j][2 * i + 1] = __builtin_fmaf(p, bf16hi_to_f32(vw[r][i]), acc[j][2 * i + 1]);
+                }
+            }
+        }
+    }
+
+    // merge the lane groups of one wave with shuffles (lanes l and l^o hold the
+    // same 8 dims of different key subsets) ...
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+        for (int j = 0; j < GROUP; j++) {
+            const float m2 = __shfl_xor(m[j], o, 64);
+            const float l2 = __shfl_xor(l[j], o, 64);
+            const float mx = fmaxf(m[j], m2);
+            const float c1 = mx > -INFINITY ? __expf(m[j] - mx) : 0.0f;
+            const float c2 = mx > -INFINITY ? __expf(m2 - mx) : 0.0f;
+            l[j] = l[j] * c1 + l2 * c2;
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                acc[j][i] = acc[j][i] * c1 + __shfl_xor(acc[j][i], o, 64) * c2;
+            m[j] = mx;
+        }
+    }
+    // ... and the waves of the workgroup through LDS
+    constexpr int NW = GQA_DEC_THREADS / 64;
+    __shared__ float sh_acc[NW][GROUP][HD];
+    __shared__ float sh_m[NW][GROUP], sh_l[NW][GROUP];
+    const int wave = tid >> 6;
+    if ((tid & 63) < LPK) {
+#pragma unroll
+        for (int j = 0; j < GROUP; j++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) sh_acc[wave][j][sub * 8 + i] = acc[j][i];
+            if (sub == 0) {
+                sh_m[wave][j] = m[j];
+                sh_l[wave][j] = l[j];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GROUP * HD; idx += GQA_DEC_THREADS) {
+        const int j = idx / HD, d = idx % HD;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; w++) mx = fmaxf(mx, sh_m[w][j]);
+        float a = 0.0f, ls = 0.0f;
+        if (mx > -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const float c = __expf(sh_m[w][j] - mx);   // exp(-inf) = 0 for idle waves
+                a += sh_acc[w][j][d] * c;
+                ls += sh_l[w][j] * c;
+            }
+        }
+        const int h = g * GROUP + j;
+        part_acc[((size_t)split * n_heads + h) * HD + d] = a;
+        if (d == 0) {
+            part_ml[((size_t)split * n_heads + h) * 2 + 0] = mx;
+            part_ml[((size_t)split * n_heads + h) * 2 + 1] = ls;
+        }
+    }
+}
+
+// out[h][d] = sum_s acc_s[h][d] e^{m_s - M} / sum_s l_s e^{m_s - M}
+template <int HD>
+__global__ void __launch_bounds__(HD)
+gqa_decode_merge_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
+                        int n_splits, int n_heads, float *__restrict__ out) {
+    const int h = blockIdx.x, d = threadIdx.x;
+    float mx = -INFINITY;
+    for (int s = 0; s < n_splits; s++) mx = fmaxf(mx, part_ml[((size_t)s * n_heads + h) * 2]);
+    float a = 0.0f, l = 0.0f;
+    for (int s = 0; s < n_splits; s++) {
+        const float ms = part_ml[((size_t)s * n_heads + h) * 2];
+        if (ms == -INFINITY) continue;
+        const float c = __expf(ms - mx);
+        a += part_acc[((size_t)s * n_heads + h) * HD + d] * c;
+        l += part_ml[((size_t)s * n_heads + h) * 2 + 1] * c;
+    }
+    out[(size_t)h * HD + d] = a / l;
+}
+
+template <int HD, int GROUP>
+static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
+                          const uint16_t *q, float scale, float *out, hipStream_t s) {
+    const int n_heads = n_kv_heads * GROUP;
+    constexpr int LPK = HD / 8, NGRP = GQA_DEC_THREADS / LPK;
+    constexpr int step = NGRP * GQA_DEC_KB;   // rows one workgroup consumes per iteration
+    // enough workgroups for ~2 per CU, each at least one full step
+    int64_t want = (int64_t)2 * num_cus() / n_kv_heads;
+    if (want < 1) want = 1;
+    int64_t per = (n_keys + want - 1) / want;
+    per = ((per + step - 1) / step) * step;
+    if (per < step) per = step;
+    const int n_splits = (int)((n_keys + per - 1) / per);
+    const size_t acc_bytes = (size_t)n_splits * n_heads * HD * sizeof(float);
+    const size_t ml_bytes = (size_t)n_splits * n_heads * 2 * sizeof(float);
+    char *ws = (char *)workspace(s, acc_bytes + ml_bytes);
+    CWICK_REQUIRE(ws, "gqa_decode: workspace allocation failed");
+    float *part_acc = (float *)ws, *part_ml = (float *)(ws + acc_bytes);
+    gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_kv_heads), GQA_DEC_THREADS, 0, s>>>(
+        k, v, q, n_keys, n_kv_heads, (int)per, scale, part_acc, part_ml);
+    CWICK_HIP_CALL(hipGetLastError());
+    gqa_decode_merge_kernel<HD><<<n_heads, HD, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
+                      int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
+                      hipStream_t s) {
+    CWICK_REQUIRE(k && v && q && out, "gqa_decode: null pointer");
+    CWICK_REQUIRE(n_keys >= 1 && n_keys <= ((int64_t)1 << 30), "gqa_decode: n_keys %lld",
+                  (long long)n_keys);
+    CWICK_REQUIRE(n_kv_heads >= 1 && n_kv_heads <= 64 && n_heads >= n_kv_heads &&
+                      n_heads % n_kv_heads == 0,
+                  "gqa_decode: n_heads %d is not a multiple of n_kv_heads %d", n_heads, n_kv_heads);
+    CWICK_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)q) % 16 == 0,
+                  "gqa_decode: K, V and q must be 16-byte aligned");
+    const int group = n_heads / n_kv_heads;
+#define CASE(HD, G)                                      \
+    if (head_dim == HD && group == G)                    \
+        return run_gqa_decode<HD, G>(k, v, n_keys, n_kv_heads, q, scale, out, s)
+    CASE(256, 1); CASE(256, 2); CASE(256, 4); CASE(256, 8);
+    CASE(128, 1); CASE(128, 2); CASE(128, 4); CASE(128, 8);
+#undef CASE
+    set_error("gqa_decode: head_dim %d with group %d is not supported (head_dim 128/256, group 1/2/4/8)",
+              head_dim, group);
+    return 0;
+}
+
+}  // namespace cwick

@@ -1,0 +1,719 @@
+// runtime.hip -- lifecycle, device-resident caches and the extern "C" surface of
+// libcwick_hip.so.  Kernels live in the other .hip files; this file only
+// validates arguments, moves host operands and enqueues.
+#include "common.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <strings.h>
+#include <unordered_map>
+
+namespace cwick {
+
+// ---------------------------------------------------------------------------
+// error text, per thread (plays the part of cwick_error.message, src/cwick.h:39-59)
+// ---------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+}
+void clear_error() { g_err[0] = 0; }
+
+bool hip_ok(hipError_t e, const char *what) {
+    if (e == hipSuccess) return true;
+    set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+    return false;
+}
+
+// ---------------------------------------------------------------------------
+// backend state machine: -1 untried, 0 unavailable, 1 ready
+// (src/h3_gpu.c:35-40, src/metal.c:22-26)
+// ---------------------------------------------------------------------------
+static std::mutex g_mu;
+static int g_state = -1;
+static int g_selected = -1;   // -1 env/auto, 0 explicit CPU, 1 explicit GPU
+static int g_cus = 0;
+static char g_info[256] = "";
+
+static int env_enabled(const char *name, int dflt) {
+    const char *v = getenv(name);
+    if (!v || !*v) return dflt;
+    return strcmp(v, "1") == 0 || strcasecmp(v, "true") == 0 || strcasecmp(v, "yes") == 0 ||
+           strcasecmp(v, "on") == 0;
+}
+
+static int bring_up_locked() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        set_error("no HIP device");
+        return 0;
+    }
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("hipGetDeviceProperties failed");
+        return 0;
+    }
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device 0 is %s; this library is built for gfx950 only", p.gcnArchName);
+        return 0;
+    }
+    if (hipSetDevice(0) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("hipSetDevice(0) failed");
+        return 0;
+    }
+    g_cus = p.multiProcessorCount;
+    snprintf(g_info, sizeof g_info, "%s %s, %d CUs, %.1f GiB, LDS %zu KiB/WG", p.name,
+             p.gcnArchName, p.multiProcessorCount,
+             (double)p.totalGlobalMem / (1024.0 * 1024.0 * 1024.0),
+             (size_t)p.sharedMemPerBlock / 1024);
+    return 1;
+}
+
+bool backend_ready() {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_state < 0) {
+        int enabled = g_selected >= 0 ? g_selected : env_enabled("CWICK_HIP", 1);
+        g_state = enabled ? bring_up_locked() : 0;
+        if (!enabled) set_error("backend not selected (CWICK_HIP=0 or cwick_hip_force(0))");
+    } else if (g_state == 0) {
+        set_error("backend unavailable or not selected");
+    }
+    return g_state == 1;
+}
+
+int num_cus() { return g_cus > 0 ? g_cus : 256; }
+
+// ---------------------------------------------------------------------------
+// grow-only scratch, one pair of buffers per stream
+// ---------------------------------------------------------------------------
+struct Scratch {
+    void *p = nullptr;
+    size_t cap = 0;
+};
+static std::unordered_map<hipStream_t, Scratch> g_ws, g_stage;
+
+static void *grow(std::unordered_map<hipStream_t, Scratch> &m, hipStream_t s, size_t bytes) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Scratch &b = m[s];
+    if (bytes <= b.cap) return b.p;
+    // A buffer in use by kernels already enqueued on `s` must outlive them.
+    if (b.p) {
+        if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize(workspace grow)")) return nullptr;
+        (void)hipFree(b.p);
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    if (!hip_ok(hipMalloc(&b.p, want), "hipMalloc(workspace)")) {
+        b.p = nullptr;
+        return nullptr;
+    }
+    b.cap = want;
+    return b.p;
+}
+
+void *workspace(hipStream_t s, size_t bytes) { return grow(g_ws, s, bytes); }
+void *staging(hipStream_t s, size_t bytes) { return grow(g_stage, s, bytes); }
+
+static void free_all_scratch() {
+    std::lock_guard<std::mutex> lk(g_mu);
+    for (auto &kv : g_ws) if (kv.second.p) (void)hipFree(kv.second.p);
+    for (auto &kv : g_stage) if (kv.second.p) (void)hipFree(kv.second.p);
+    g_ws.clear();
+    g_stage.clear();
+}
+
+}  // namespace cwick
+
+using namespace cwick;
+
+// ---------------------------------------------------------------------------
+// cache handles
+// ---------------------------------------------------------------------------
+struct cwick_hip_kv {
+    int64_t capacity;
+    int n_kv_heads, head_dim;
+    uint16_t *k, *v;
+};
+struct cwick_hip_latent {
+    int slots;
+    int64_t capacity;
+    uint8_t *rows;    // [slots][capacity][576]
+    float *scales;    // [slots][capacity][5]
+};
+struct cwick_hip_ikeys {
+    int slots;
+    int64_t capacity;
+    uint8_t *rows;    // [slots][capacity][128]
+    float *scales;    // [slots][capacity]
+};
+
+// Stage `bytes` of host memory into the per-stream staging buffer at `off`.
+static void *stage_in(char *base, size_t &off, const void *host, size_t bytes) {
+    void *d = base + off;
+    off += (bytes + 255) & ~(size_t)255;
+    if (hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, nullptr) != hipSuccess) return nullptr;
+    return d;
+}
+static size_t pad256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+extern "C" {
+
+// ---- lifecycle -------------------------------------------------------------
+int cwick_hip_ready(void) {
+    clear_error();
+    return backend_ready() ? 1 : 0;
+}
+
+int cwick_hip_force(int on) {
+    clear_error();
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        g_selected = on ? 1 : 0;
+        g_state = on ? -1 : 0;
+    }
+    if (!on) return 0;
+    return backend_ready() ? 0 : -1;
+}
+
+void cwick_hip_shutdown(void) {
+    if (g_state == 1) (void)hipDeviceSynchronize();
+    free_all_scratch();
+}
+
+const char *cwick_hip_last_error(void) { return g_err; }
+
+int cwick_hip_device_info(char *buf, size_t cap) {
+    clear_error();
+    if (!backend_ready() || !buf || cap == 0) return 0;
+    snprintf(buf, cap, "%s", g_info);
+    return 1;
+}
+
+// ---- GQA cache -------------------------------------------------------------
+cwick_hip_kv *cwick_hip_kv_create(int64_t capacity, int n_kv_heads, int head_dim) {
+    clear_error();
+    if (!backend_ready()) return nullptr;
+    if (capacity <= 0 || n_kv_heads <= 0 || (head_dim != 128 && head_dim != 256)) {
+        set_error("kv_create: capacity %lld, n_kv_heads %d, head_dim %d unsupported",
+                  (long long)capacity, n_kv_heads, head_dim);
+        return nullptr;
+    }
+    cwick_hip_kv *c = new cwick_hip_kv{capacity, n_kv_heads, head_dim, nullptr, nullptr};
+    size_t bytes = (size_t)capacity * n_kv_heads * head_dim * sizeof(uint16_t);
+    if (!hip_ok(hipMalloc((void **)&c->k, bytes), "hipMalloc(K cache)") ||
+        !hip_ok(hipMalloc((void **)&c->v, bytes), "hipMalloc(V cache)")) {
+        if (c->k) (void)hipFree(c->k);
+        delete c;
+        return nullptr;
+    }
+    return c;
+}
+
+void cwick_hip_kv_free(cwick_hip_kv *c) {
+    if (!c) return;
+    (void)hipDeviceSynchronize();
+    (void)hipFree(c->k);
+    (void)hipFree(c->v);
+    delete c;
+}
+
+int cwick_hip_kv_write(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *k_rows,
+                       const uint16_t *v_rows) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && k_rows && v_rows, "kv_write: null argument");
+    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,
+                  "kv_write: rows %lld..%lld outside capacity %lld", (long long)pos0,
+                  (long long)(pos0 + n), (long long)c->capacity);
+    size_t row = (size_t)c->n_kv_heads * c->head_dim;
+    CWICK_HIP_CALL(hipMemcpy(c->k + pos0 * row, k_rows, n * row * 2, hipMemcpyHostToDevice));
+    CWICK_HIP_CALL(hipMemcpy(c->v + pos0 * row, v_rows, n * row * 2, hipMemcpyHostToDevice));
+    return 1;
+}
+
+int cwick_hip_kv_write_f32(cwick_hip_kv *c, int64_t pos0, int64_t n, const float *k_rows,
+                           const float *v_rows) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && k_rows && v_rows, "kv_write_f32: null argument");
+    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,
+                  "kv_write_f32: rows outside capacity");
+    size_t row = (size_t)c->n_kv_heads * c->head_dim;
+    size_t bytes = (size_t)n * row * sizeof(float);
+    char *st = (char *)staging(nullptr, 2 * pad256(bytes));
+    CWICK_REQUIRE(st, "kv_write_f32: staging allocation failed");
+    size_t off = 0;
+    float *dk = (float *)stage_in(st, off, k_rows, bytes);
+    float *dv = (float *)stage_in(st, off, v_rows, bytes);
+    CWICK_REQUIRE(dk && dv, "kv_write_f32: upload failed");
+    if (!launch_narrow_bf16(dk, n * row, c->k + pos0 * row, nullptr)) return 0;
+    if (!launch_narrow_bf16(dv, n * row, c->v + pos0 * row, nullptr)) return 0;
+    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
+    return 1;
+}
+
+uint16_t *cwick_hip_kv_k_dev(cwick_hip_kv *c) { return c ? c->k : nullptr; }
+uint16_t *cwick_hip_kv_v_dev(cwick_hip_kv *c) { return c ? c->v : nullptr; }
+
+// ---- latent cache ------------------------------------------------------------
+cwick_hip_latent *cwick_hip_latent_create(int slots, int64_t capacity) {
+    clear_error();
+    if (!backend_ready()) return nullptr;
+    if (slots <= 0 || capacity <= 0) {
+        set_error("latent_create: slots %d capacity %lld", slots, (long long)capacity);
+        return nullptr;
+    }
+    cwick_hip_latent *c = new cwick_hip_latent{slots, capacity, nullptr, nullptr};
+    size_t rows = (size_t)slots * capacity;
+    // 64 bytes of slack: the kernels read rows in 16-byte pieces
+    if (!hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_LATENT_KDIM + 64), "hipMalloc(latent)") ||
+        !hip_ok(hipMalloc((void **)&c->scales, rows * CWICK_HIP_LATENT_NBLK * sizeof(float) + 64),
+                "hipMalloc(latent scales)")) {
+        if (c->rows) (void)hipFree(c->rows);
+        delete c;
+        return nullptr;
+    }
+    return c;
+}
+
+void cwick_hip_latent_free(cwick_hip_latent *c) {
+    if (!c) return;
+    (void)hipDeviceSynchronize();
+    (void)hipFree(c->rows);
+    (void)hipFree(c->scales);
+    delete c;
+}
+
+#define LATENT_RANGE_CHECK(what)                                                          \
+    CWICK_REQUIRE(backend_ready(), "backend not ready");                                  \
+    CWICK_REQUIRE(c, what ": null handle");                                               \
+    CWICK_REQUIRE(slot >= 0 && slot < c->slots, what ": slot %d of %d", slot, c->slots);  \
+    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,                          \
+                  what ": rows %lld..%lld outside capacity %lld", (long long)pos0,       \
+                  (long long)(pos0 + n), (long long)c->capacity)
+
+int cwick_hip_latent_write(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                           const uint8_t *rows, const float *scales) {
+    clear_error();
+    LATENT_RANGE_CHECK("latent_write");
+    CWICK_REQUIRE(rows && scales, "latent_write: null argument");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    CWICK_HIP_CALL(hipMemcpy(c->rows + r0 * CWICK_HIP_LATENT_KDIM, rows,
+                             (size_t)n * CWICK_HIP_LATENT_KDIM, hipMemcpyHostToDevice));
+    CWICK_HIP_CALL(hipMemcpy(c->scales + r0 * CWICK_HIP_LATENT_NBLK, scales,
+                             (size_t)n * CWICK_HIP_LATENT_NBLK * sizeof(float),
+                             hipMemcpyHostToDevice));
+    return 1;
+}
+
+int cwick_hip_latent_write_f32(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                               const float *rows) {
+    clear_error();
+    LATENT_RANGE_CHECK("latent_write_f32");
+    CWICK_REQUIRE(rows, "latent_write_f32: null argument");
+    size_t bytes = (size_t)n * CWICK_HIP_LATENT_KDIM * sizeof(float);
+    char *st = (char *)staging(nullptr, pad256(bytes));
+    CWICK_REQUIRE(st, "latent_write_f32: staging allocation failed");
+    size_t off = 0;
+    float *d = (float *)stage_in(st, off, rows, bytes);
+    CWICK_REQUIRE(d, "latent_write_f32: upload failed");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    if (!launch_quant_latent(d, n, c->rows + r0 * CWICK_HIP_LATENT_KDIM,
+                             c->scales + r0 * CWICK_HIP_LATENT_NBLK, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
+    return 1;
+}
+
+int cwick_hip_latent_read(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n, uint8_t *rows,
+                          float *scales) {
+    clear_error();
+    LATENT_RANGE_CHECK("latent_read");
+    CWICK_REQUIRE(rows && scales, "latent_read: null argument");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    CWICK_HIP_CALL(hipMemcpy(rows, c->rows + r0 * CWICK_HIP_LATENT_KDIM,
+                             (size_t)n * CWICK_HIP_LATENT_KDIM, hipMemcpyDeviceToHost));
+    CWICK_HIP_CALL(hipMemcpy(scales, c->scales + r0 * CWICK_HIP_LATENT_NBLK,
+                             (size_t)n * CWICK_HIP_LATENT_NBLK * sizeof(float),
+                             hipMemcpyDeviceToHost));
+    return 1;
+}
+
+uint8_t *cwick_hip_latent_rows_dev(cwick_hip_latent *c, int slot) {
+    if (!c || slot < 0 || slot >= c->slots) return nullptr;
+    return c->rows + (size_t)slot * c->capacity * CWICK_HIP_LATENT_KDIM;
+}
+float *cwick_hip_latent_scales_dev(cwick_hip_latent *c, int slot) {
+    if (!c || slot < 0 || slot >= c->slots) return nullptr;
+    return c->scales + (size_t)slot * c->capacity * CWICK_HIP_LATENT_NBLK;
+}
+
+// ---- indexer key cache -------------------------------------------------------
+cwick_hip_ikeys *cwick_hip_ikeys_create(int slots, int64_t capacity) {
+    clear_error();
+    if (!backend_ready()) return nullptr;
+    if (slots <= 0 || capacity <= 0) {
+        set_error("ikeys_create: slots %d capacity %lld", slots, (long long)capacity);
+        return nullptr;
+    }
+    cwick_hip_ikeys *c = new cwick_hip_ikeys{slots, capacity, nullptr, nullptr};
+    size_t rows = (size_t)slots * capacity;
+    if (!hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_INDEX_DIM + 64), "hipMalloc(ikeys)") ||
+        !hip_ok(hipMalloc((void **)&c->scales, rows * sizeof(float) + 64), "hipMalloc(ikey scales)")) {
+        if (c->rows) (void)hipFree(c->rows);
+        delete c;
+        return nullptr;
+    }
+    return c;
+}
+
+void cwick_hip_ikeys_free(cwick_hip_ikeys *c) {
+    if (!c) return;
+    (void)hipDeviceSynchronize();
+    (void)hipFree(c->rows);
+    (void)hipFree(c->scales);
+    delete c;
+}
+
+int cwick_hip_ikeys_write(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
+                          const uint8_t *rows, const float *scales) {
+    clear_error();
+    LATENT_RANGE_CHECK("ikeys_write");
+    CWICK_REQUIRE(rows && scales, "ikeys_write: null argument");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    CWICK_HIP_CALL(hipMemcpy(c->rows + r0 * CWICK_HIP_INDEX_DIM, rows,
+                             (size_t)n * CWICK_HIP_INDEX_DIM, hipMemcpyHostToDevice));
+    CWICK_HIP_CALL(hipMemcpy(c->scales + r0, scales, (size_t)n * sizeof(float),
+                             hipMemcpyHostToDevice));
+    return 1;
+}
+
+int cwick_hip_ikeys_write_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
+                              const float *rows) {
+    clear_error();
+    LATENT_RANGE_CHECK("ikeys_write_f32");
+    CWICK_REQUIRE(rows, "ikeys_write_f32: null argument");
+    size_t bytes = (size_t)n * CWICK_HIP_INDEX_DIM * sizeof(float);
+    char *st = (char *)staging(nullptr, pad256(bytes));
+    CWICK_REQUIRE(st, "ikeys_write_f32: staging allocation failed");
+    size_t off = 0;
+    float *d = (float *)stage_in(st, off, rows, bytes);
+    CWICK_REQUIRE(d, "ikeys_write_f32: upload failed");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    if (!launch_quant_ikeys(d, n, c->rows + r0 * CWICK_HIP_INDEX_DIM, c->scales + r0, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
+    return 1;
+}
+
+uint8_t *cwick_hip_ikeys_rows_dev(cwick_hip_ikeys *c, int slot) {
+    if (!c || slot < 0 || slot >= c->slots) return nullptr;
+    return c->rows + (size_t)slot * c->capacity * CWICK_HIP_INDEX_DIM;
+}
+float *cwick_hip_ikeys_scales_dev(cwick_hip_ikeys *c, int slot) {
+    if (!c || slot < 0 || slot >= c->slots) return nullptr;
+    return c->scales + (size_t)slot * c->capacity;
+}
+
+// ---- device-pointer entry points ---------------------------------------------
+int cwick_hip_gqa_decode_dev(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
+                             int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
+                             void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_gqa_decode(k, v, n_keys, n_kv_heads, head_dim, q, n_heads, scale, out,
+                             (hipStream_t)stream);
+}
+
+int cwick_hip_gqa_prefill_dev(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
+                              int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
+                              float scale, float *out, void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_gqa_prefill(k, v, pos0, n, n_kv_heads, head_dim, q, n_heads, scale, out,
+                              (hipStream_t)stream);
+}
+
+int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales, int64_t row_batch_stride,
+                             int64_t scale_batch_stride, int64_t n_rows, int batch, const int32_t *sel,
+                             int64_t n_list, const uint16_t *q, int n_heads, float scale,
+                             float *out, void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_rows, batch, sel,
+                             n_list, q, n_heads, scale, out, (hipStream_t)stream);
+}
+
+int cwick_hip_mla_prefill_chunk_dev(const uint8_t *rows, const float *scales, int64_t pos0,
+                                    int64_t n, const uint16_t *q, int n_heads, float scale,
+                                    float *out, void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_mla_prefill(rows, scales, pos0, n, q, n_heads, scale, out, (hipStream_t)stream);
+}
+
+int cwick_hip_indexer_scores_dev(const uint8_t *keys, const float *kscale, int64_t key_batch_stride,
+                                 int64_t kscale_batch_stride, int batch, int64_t n_keys,
+                                 const uint16_t *q_idx, const float *w, int n_idx_heads,
+                                 float *scores, void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_indexer_scores(keys, kscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
+                                 q_idx, w, n_idx_heads, scores, (hipStream_t)stream);
+}
+
+int cwick_hip_topk_dev(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
+                       void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    return launch_topk(scores, batch, n, k, out_idx, (hipStream_t)stream);
+}
+
+int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale, int64_t key_batch_stride,
+                             int64_t kscale_batch_stride, const uint8_t *rows, const float *scales,
+                             int64_t row_batch_stride, int64_t scale_batch_stride, int batch,
+                             int64_t n_keys, const uint16_t *q_idx, const float *w, int n_idx_heads,
+                             int64_t topk, const uint16_t *q, int n_heads, float scale,
+                             float *scores_tmp, int32_t *sel_out, float *out, void *stream) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(scores_tmp && sel_out, "dsa_decode_dev: scores_tmp and sel_out are required");
+    CWICK_REQUIRE(topk > 0 && n_keys > 0, "dsa_decode_dev: topk %lld n_keys %lld",
+                  (long long)topk, (long long)n_keys);
+    hipStream_t s = (hipStream_t)stream;
+    if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
+                               q_idx, w, n_idx_heads, scores_tmp, s))
+        return 0;
+    if (!launch_topk(scores_tmp, batch, n_keys, topk, sel_out, s)) return 0;
+    // rows past min(topk, n_keys) are -1 and are skipped by the attention kernel
+    return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_keys, batch,
+                             sel_out, topk, q, n_heads, scale, out, s);
+}
+
+// ---- host-pointer entry points -------------------------------------------------
+int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q, int n_heads,
+                         float scale, float *out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q && out, "gqa_decode: null argument");
+    CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "gqa_decode: n_keys %lld, capacity %lld",
+                  (long long)n_keys, (long long)c->capacity);
+    CWICK_REQUIRE(n_heads > 0 && n_heads <= 1024, "gqa_decode: n_heads %d", n_heads);
+    size_t qb = (size_t)n_heads * c->head_dim * 2, ob = (size_t)n_heads * c->head_dim * 4;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st, "gqa_decode: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    CWICK_REQUIRE(dq, "gqa_decode: upload failed");
+    float *dout = (float *)(st + off);
+    if (!launch_gqa_decode(c->k, c->v, n_keys, c->n_kv_heads, c->head_dim, dq, n_heads, scale, dout,
+                           nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *q, int n_heads,
+                          float scale, float *out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q && out, "gqa_prefill: null argument");
+    CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= c->capacity,
+                  "gqa_prefill: positions %lld..%lld outside capacity %lld", (long long)pos0,
+                  (long long)(pos0 + n), (long long)c->capacity);
+    CWICK_REQUIRE(n_heads > 0 && n_heads <= 1024, "gqa_prefill: n_heads %d", n_heads);
+    size_t qb = (size_t)n * n_heads * c->head_dim * 2, ob = (size_t)n * n_heads * c->head_dim * 4;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st, "gqa_prefill: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    CWICK_REQUIRE(dq, "gqa_prefill: upload failed");
+    float *dout = (float *)(st + off);
+    if (!launch_gqa_prefill(c->k, c->v, pos0, n, c->n_kv_heads, c->head_dim, dq, n_heads, scale,
+                            dout, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+// sel entries must address rows of the slot; checked on the host because a bad
+// index would be an out-of-bounds read on the device.
+static int check_sel(const int32_t *sel, int64_t n, int64_t capacity) {
+    for (int64_t i = 0; i < n; i++)
+        if (sel[i] >= capacity) {
+            set_error("sel[%lld] = %d is outside capacity %lld", (long long)i, sel[i],
+                      (long long)capacity);
+            return 0;
+        }
+    return 1;
+}
+
+int cwick_hip_mla_decode(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
+                         const uint16_t *q, int n_heads, float scale, float *out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q && out, "mla_decode: null argument");
+    CWICK_REQUIRE(slot >= 0 && slot < c->slots, "mla_decode: slot %d of %d", slot, c->slots);
+    CWICK_REQUIRE(n_list >= 1, "mla_decode: n_list %lld", (long long)n_list);
+    CWICK_REQUIRE(sel || n_list <= c->capacity, "mla_decode: n_list %lld > capacity %lld",
+                  (long long)n_list, (long long)c->capacity);
+    CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
+    if (sel && !check_sel(sel, n_list, c->capacity)) return 0;
+    size_t qb = (size_t)n_heads * CWICK_HIP_LATENT_KDIM * 2;
+    size_t ob = (size_t)n_heads * CWICK_HIP_LATENT_VDIM * 4;
+    size_t sb = sel ? (size_t)n_list * 4 : 0;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob) + pad256(sb));
+    CWICK_REQUIRE(st, "mla_decode: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    int32_t *dsel = sel ? (int32_t *)stage_in(st, off, sel, sb) : nullptr;
+    CWICK_REQUIRE(dq && (!sel || dsel), "mla_decode: upload failed");
+    float *dout = (float *)(st + off);
+    if (!launch_mla_decode(cwick_hip_latent_rows_dev(c, slot), cwick_hip_latent_scales_dev(c, slot),
+                           0, 0, c->capacity, 1, dsel, n_list, dq, n_heads, scale, dout, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+int cwick_hip_mla_prefill_chunk(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                                const uint16_t *q, int n_heads, float scale, float *out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q && out, "mla_prefill_chunk: null argument");
+    CWICK_REQUIRE(slot >= 0 && slot < c->slots, "mla_prefill_chunk: slot %d of %d", slot, c->slots);
+    CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= c->capacity,
+                  "mla_prefill_chunk: positions %lld..%lld outside capacity %lld", (long long)pos0,
+                  (long long)(pos0 + n), (long long)c->capacity);
+    CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill_chunk: n_heads %d (1..128)", n_heads);
+    size_t qb = (size_t)n * n_heads * CWICK_HIP_LATENT_KDIM * 2;
+    size_t ob = (size_t)n * n_heads * CWICK_HIP_LATENT_VDIM * 4;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st, "mla_prefill_chunk: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    CWICK_REQUIRE(dq, "mla_prefill_chunk: upload failed");
+    float *dout = (float *)(st + off);
+    if (!launch_mla_prefill(cwick_hip_latent_rows_dev(c, slot), cwick_hip_latent_scales_dev(c, slot),
+                            pos0, n, dq, n_heads, scale, dout, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys, const uint16_t *q_idx,
+                             const float *w, int n_idx_heads, float *scores) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q_idx && w && scores, "indexer_scores: null argument");
+    CWICK_REQUIRE(slot >= 0 && slot < c->slots, "indexer_scores: slot %d of %d", slot, c->slots);
+    CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "indexer_scores: n_keys %lld, capacity %lld",
+                  (long long)n_keys, (long long)c->capacity);
+    CWICK_REQUIRE(n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_scores: n_idx_heads %d (1..64)",
+                  n_idx_heads);
+    size_t qb = (size_t)n_idx_heads * CWICK_HIP_INDEX_DIM * 2, wb = (size_t)n_idx_heads * 4;
+    size_t ob = (size_t)n_keys * 4;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(wb) + pad256(ob));
+    CWICK_REQUIRE(st, "indexer_scores: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q_idx, qb);
+    float *dw = (float *)stage_in(st, off, w, wb);
+    CWICK_REQUIRE(dq && dw, "indexer_scores: upload failed");
+    float *dout = (float *)(st + off);
+    if (!launch_indexer_scores(cwick_hip_ikeys_rows_dev(c, slot), cwick_hip_ikeys_scales_dev(c, slot),
+                               0, 0, 1, n_keys, dq, dw, n_idx_heads, dout, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(scores, dout, ob, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+int cwick_hip_topk(const float *scores, int64_t n, int64_t k, int32_t *out_idx, int64_t *n_out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(scores && out_idx, "topk: null argument");
+    CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
+    CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
+    size_t sb = (size_t)n * 4, ob = (size_t)k * 4;
+    char *st = (char *)staging(nullptr, pad256(sb) + pad256(ob));
+    CWICK_REQUIRE(st, "topk: staging allocation failed");
+    size_t off = 0;
+    float *ds = (float *)stage_in(st, off, scores, sb);
+    CWICK_REQUIRE(ds, "topk: upload failed");
+    int32_t *dout = (int32_t *)(st + off);
+    if (!launch_topk(ds, 1, n, k, dout, nullptr)) return 0;
+    int64_t got = k < n ? k : n;
+    CWICK_HIP_CALL(hipMemcpy(out_idx, dout, (size_t)got * 4, hipMemcpyDeviceToHost));
+    if (n_out) *n_out = got;
+    return 1;
+}
+
+int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, int slot_step,
+                         int batch, int64_t n_keys, const uint16_t *q_idx, const float *w,
+                         int n_idx_heads, int64_t topk, const uint16_t *q, int n_heads, float scale,
+                         float *out, int32_t *sel_out) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(ik && lat && q_idx && w && q && out, "dsa_decode: null argument");
+    CWICK_REQUIRE(batch >= 1 && batch <= 1024, "dsa_decode: batch %d", batch);
+    CWICK_REQUIRE(slot_step == 0 || slot_step == 1, "dsa_decode: slot_step %d (0 or 1)", slot_step);
+    int last = slot0 + (batch - 1) * slot_step;
+    CWICK_REQUIRE(slot0 >= 0 && last < ik->slots && last < lat->slots,
+                  "dsa_decode: slots %d..%d outside the caches", slot0, last);
+    CWICK_REQUIRE(n_keys >= 1 && n_keys <= ik->capacity && n_keys <= lat->capacity,
+                  "dsa_decode: n_keys %lld exceeds a cache capacity", (long long)n_keys);
+    CWICK_REQUIRE(n_idx_heads >= 1 && n_idx_heads <= 64, "dsa_decode: n_idx_heads %d", n_idx_heads);
+    CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "dsa_decode: n_heads %d", n_heads);
+    CWICK_REQUIRE(topk >= 1 && topk <= 65536, "dsa_decode: topk %lld", (long long)topk);
+    size_t qib = (size_t)batch * n_idx_heads * CWICK_HIP_INDEX_DIM * 2;
+    size_t wb = (size_t)batch * n_idx_heads * 4;
+    size_t qb = (size_t)batch * n_heads * CWICK_HIP_LATENT_KDIM * 2;
+    size_t scb = (size_t)batch * n_keys * 4, selb = (size_t)batch * topk * 4;
+    size_t ob = (size_t)batch * n_heads * CWICK_HIP_LATENT_VDIM * 4;
+    char *st = (char *)staging(nullptr, pad256(qib) + pad256(wb) + pad256(qb) + pad256(scb) +
+                                            pad256(selb) + pad256(ob));
+    CWICK_REQUIRE(st, "dsa_decode: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dqi = (uint16_t *)stage_in(st, off, q_idx, qib);
+    float *dw = (float *)stage_in(st, off, w, wb);
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    CWICK_REQUIRE(dqi && dw && dq, "dsa_decode: upload failed");
+    float *dsc = (float *)(st + off); off += pad256(scb);
+    int32_t *dsel = (int32_t *)(st + off); off += pad256(selb);
+    float *dout = (float *)(st + off);
+    int ok = cwick_hip_dsa_decode_dev(
+        cwick_hip_ikeys_rows_dev(ik, slot0), cwick_hip_ikeys_scales_dev(ik, slot0),
+        (int64_t)slot_step * ik->capacity * CWICK_HIP_INDEX_DIM, (int64_t)slot_step * ik->capacity,
+        cwick_hip_latent_rows_dev(lat, slot0), cwick_hip_latent_scales_dev(lat, slot0),
+        (int64_t)slot_step * lat->capacity * CWICK_HIP_LATENT_KDIM,
+        (int64_t)slot_step * lat->capacity * CWICK_HIP_LATENT_NBLK, batch, n_keys, dqi, dw,
+        n_idx_heads, topk, dq, n_heads, scale, dsc, dsel, dout, nullptr);
+    if (!ok) return 0;
+    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
+    if (sel_out) CWICK_HIP_CALL(hipMemcpy(sel_out, dsel, selb, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+int cwick_hip_e4m3_table(float *out256) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(out256, "e4m3_table: null argument");
+    float *d = (float *)staging(nullptr, 1024);
+    CWICK_REQUIRE(d, "e4m3_table: staging allocation failed");
+    if (!launch_e4m3_table(d, nullptr)) return 0;
+    CWICK_HIP_CALL(hipMemcpy(out256, d, 1024, hipMemcpyDeviceToHost));
+    return 1;
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+// topk.hip -- exact top-k by radix select (ds_topk_scores, src/ds_ops.c:310-338,
+// under the contract of src/ds_ops.h:110-112; the threshold-then-ties selector
+// of src/attention.c:585-598 computes the same set).
+//
+// Order: (score descending, index ascending); the k best are written in
+// ascending index order.  Scores map to order-preserving 32-bit keys
+// (-0.0 folded into +0.0, NaN below everything), so the selection is integer
+// work and bit-exact by construction:
+//
+//   1. four 8-bit histogram passes, most significant digit first, find the key
+//      T of the k-th best element and r = how many elements equal to T belong
+//      to the selection;
+//   2. one ordered pass emits every index with key > T and the first r indices
+//      with key == T, in ascending index order, through a block-wide scan.
+//
+// One workgroup of 1024 threads per batch row; the row (n * 4 bytes) is read
+// five times from L2.  Rows past min(k, n) are filled with -1.
+#include "common.hpp"
+
+namespace cwick {
+
+constexpr int TOPK_THREADS = 1024;
+constexpr int TOPK_WAVES = TOPK_THREADS / 64;
+
+__device__ __forceinline__ uint32_t topk_key(float f) {
+    if (f != f) return 0u;
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u << 1) == 0u) u = 0u;                       // -0.0 -> +0.0
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return u == 0u ? 1u : u;
+}
+
+// exclusive scan of one value per thread across the block; returns the
+// exclusive prefix and writes the block total to *total
+__device__ __forceinline__ uint32_t block_exscan(uint32_t v, uint32_t *sh_wave, uint32_t *total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        uint32_t t = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += t;
+    }
+    if (lane == 63) sh_wave[wave] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < TOPK_WAVES; w++) {
+        const uint32_t c = sh_wave[w];
+        if (w < wave) wave_off += c;
+        tot += c;
+    }
+    __syncthreads();
+    *total = tot;
+    return wave_off + inc - v;
+}
+
+__global__ void __launch_bounds__(TOPK_THREADS)
+topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
+                  int32_t *__restrict__ out) {
+    // 16 copies of the histogram, picked by lane, so that the lanes of a wave
+    // that hit one digit (scores cluster in a few exponent buckets) do not all
+    // serialise on one LDS word
+    __shared__ uint32_t hist16[256 * 16];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t sh_wave[TOPK_WAVES];
+    __shared__ uint32_t sh_prefix, sh_remaining;
+    const float *sc = scores + (size_t)blockIdx.x * n;
+    int32_t *dst = out + (size_t)blockIdx.x * k;
+    const int tid = threadIdx.x;
+    const int64_t kk = k < n ? k : n;
+
+    for (int64_t i = kk + tid; i < k; i += TOPK_THREADS) dst[i] = -1;
+
+    if (tid == 0) {
+        sh_prefix = 0u;
+        sh_remaining = (uint32_t)kk;
+    }
+    // ---- 1. find the key of the kk-th best element ----
+    uint32_t prefix = 0u, mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) hist16[tid * 4 + j] = 0u;
+        __syncthreads();
+        for (int64_t i = tid; i < n; i += TOPK_THREADS) {
+            const uint32_t key = topk_key(sc[i]);
+            if ((key & mask) == prefix)
+                atomicAdd(&hist16[((key >> shift) & 0xFFu) * 16 + (tid & 15)], 1u);
+        }
+        __syncthreads();
+        if (tid < 256) {
+            uint32_t c = 0u;
+#pragma unroll
+            for (int j = 0; j < 16; j++) c += hist16[tid * 16 + j];
+            hist[tid] = c;
+        }
+        __syncthreads();
+        if (tid < 64) {
+            // walk the 256 buckets from the largest digit down; lane b owns
+            // buckets 255-4b .. 252-4b
+            const uint32_t remaining = sh_remaining;
+            uint32_t c[4], sum = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                c[j] = hist[255 - (tid * 4 + j)];
+                sum += c[j];
+            }
+            uint32_t inc = sum;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                uint32_t t = __shfl_up(inc, o, 64);
+                if (tid >= o) inc += t;
+            }
+            uint32_t before = inc - sum;   // elements in strictly larger buckets
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (before < remaining && remaining <= before + c[j]) {
+                    sh_prefix = prefix | ((uint32_t)(255 - (tid * 4 + j)) << shift);
+                    sh_remaining = remaining - before;
+                }
+                before += c[j];
+            }
+        }
+        __syncthreads();
+        prefix = sh_prefix;
+        mask |= 0xFFu << shift;
+    }
+    const uint32_t T = prefix;
+    const uint32_t r = sh_remaining;   // elements equal to T that belong to the selection
+
+    // ---- 2. ordered emit ----
+    uint32_t out_base = 0u, eq_base = 0u;
+    for (int64_t base = 0; base < n; base += (int64_t)TOPK_THREADS * 4) {
+        const int64_t i0 = base + (int64_t)tid * 4;
+        uint32_t key[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) key[j] = (i0 + j < n) ? topk_key(sc[i0 + j]) : 0u;
+        uint32_t n_eq = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; j++) n_eq += (i0 + j < n && key[j] == T) ? 1u : 0u;
+        uint32_t eq_total;
+        uint32_t eq_before = eq_base + block_exscan(n_eq, sh_wave, &eq_total);
+        uint32_t take[4], n_take = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool in = i0 + j < n;
+            const bool gt = in && key[j] > T;
+            const bool eq = in && key[j] == T;
+            take[j] = (gt || (eq && eq_before < r)) ? 1u : 0u;
+            if (eq) eq_before++;
+            n_take += take[j];
+        }
+        uint32_t take_total;
+        uint32_t pos = out_base + block_exscan(n_take, sh_wave, &take_total);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (take[j]) dst[pos++] = (int32_t)(i0 + j);
+        out_base += take_total;
+        eq_base += eq_total;
+    }
+}
+
+int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
+                hipStream_t s) {
+    CWICK_REQUIRE(scores && out_idx, "topk: null pointer");
+    CWICK_REQUIRE(batch >= 1 && batch <= 65535, "topk: batch %d", batch);
+    CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
+    CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
+    topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+}  // namespace cwick

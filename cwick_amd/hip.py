@@ -1,0 +1,398 @@
+"""ctypes binding of libcwick_hip.so (include/cwick_hip.h), one Python function
+per C entry point with the same name, argument meaning and 1/0 convention.
+
+There is no CPU fallback here: if the library is missing the import of any
+function raises, and a call that the library declines raises Declined with the
+library's own reason (cwick_hip_last_error) unless the caller asks for the raw
+return code.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcwick_hip.so")
+
+KDIM, VDIM, NBLK, BLOCK, IDIM = 576, 512, 5, 128, 128
+
+
+class Declined(RuntimeError):
+    """The GPU backend returned 0: the engine would run its CPU path."""
+
+
+_lib = None
+
+_u8p, _u16p, _i32p, _f32p = (C.POINTER(C.c_uint8), C.POINTER(C.c_uint16),
+                             C.POINTER(C.c_int32), C.POINTER(C.c_float))
+_vp, _i64, _int, _flt = C.c_void_p, C.c_int64, C.c_int, C.c_float
+
+# name -> (restype, argtypes); every symbol include/cwick_hip.h declares
+SIGNATURES = {
+    "cwick_hip_ready": (_int, []),
+    "cwick_hip_force": (_int, [_int]),
+    "cwick_hip_shutdown": (None, []),
+    "cwick_hip_last_error": (C.c_char_p, []),
+    "cwick_hip_device_info": (_int, [C.c_char_p, C.c_size_t]),
+    "cwick_hip_kv_create": (_vp, [_i64, _int, _int]),
+    "cwick_hip_kv_free": (None, [_vp]),
+    "cwick_hip_kv_write": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "cwick_hip_kv_write_f32": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "cwick_hip_kv_k_dev": (_vp, [_vp]),
+    "cwick_hip_kv_v_dev": (_vp, [_vp]),
+    "cwick_hip_latent_create": (_vp, [_int, _i64]),
+    "cwick_hip_latent_free": (None, [_vp]),
+    "cwick_hip_latent_write": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
+    "cwick_hip_latent_write_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
+    "cwick_hip_latent_read": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
+    "cwick_hip_latent_rows_dev": (_vp, [_vp, _int]),
+    "cwick_hip_latent_scales_dev": (_vp, [_vp, _int]),
+    "cwick_hip_ikeys_create": (_vp, [_int, _i64]),
+    "cwick_hip_ikeys_free": (None, [_vp]),
+    "cwick_hip_ikeys_write": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
+    "cwick_hip_ikeys_write_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
+    "cwick_hip_ikeys_rows_dev": (_vp, [_vp, _int]),
+    "cwick_hip_ikeys_scales_dev": (_vp, [_vp, _int]),
+    "cwick_hip_gqa_decode": (_int, [_vp, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_gqa_prefill": (_int, [_vp, _i64, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_mla_decode": (_int, [_vp, _int, _vp, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_mla_prefill_chunk": (_int, [_vp, _int, _i64, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_indexer_scores": (_int, [_vp, _int, _i64, _vp, _vp, _int, _vp]),
+    "cwick_hip_topk": (_int, [_vp, _i64, _i64, _vp, C.POINTER(_i64)]),
+    "cwick_hip_dsa_decode": (_int, [_vp, _vp, _int, _int, _int, _i64, _vp, _vp, _int, _i64,
+                                    _vp, _int, _flt, _vp, _vp]),
+    "cwick_hip_gqa_decode_dev": (_int, [_vp, _vp, _i64, _int, _int, _vp, _int, _flt, _vp, _vp]),
+    "cwick_hip_gqa_prefill_dev": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp, _int, _flt,
+                                         _vp, _vp]),
+    "cwick_hip_mla_decode_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
+                                        _flt, _vp, _vp]),
+    "cwick_hip_mla_prefill_chunk_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _flt, _vp, _vp]),
+    "cwick_hip_indexer_scores_dev": (_int, [_vp, _vp, _i64, _i64, _int, _i64, _vp, _vp, _int,
+                                            _vp, _vp]),
+    "cwick_hip_topk_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
+    "cwick_hip_dsa_decode_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _int, _i64,
+                                        _vp, _vp, _int, _i64, _vp, _int, _flt, _vp, _vp, _vp,
+                                        _vp]),
+    "cwick_hip_e4m3_table": (_int, [_vp]),
+}
+
+
+def lib():
+    """Load libcwick_hip.so.  Raises if it has not been built: nothing in this
+    package computes attention any other way."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: build it with `python -m cwick_amd.build` (hipcc, gfx950)"
+                % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().cwick_hip_last_error().decode("utf-8", "replace")
+
+
+def _check(rc, what):
+    if rc != 1:
+        raise Declined("%s declined: %s" % (what, last_error()))
+    return rc
+
+
+def ready():
+    return lib().cwick_hip_ready() == 1
+
+
+def force(on):
+    return lib().cwick_hip_force(1 if on else 0)
+
+
+def shutdown():
+    lib().cwick_hip_shutdown()
+
+
+def device_info():
+    buf = C.create_string_buffer(256)
+    if lib().cwick_hip_device_info(buf, 256) != 1:
+        raise Declined("device_info: " + last_error())
+    return buf.value.decode()
+
+
+def _np(a, dtype):
+    a = np.ascontiguousarray(a, dtype)
+    return a, a.ctypes.data
+
+
+def _dp(t):
+    """Device address of a torch tensor (or a raw integer address / None)."""
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    assert t.is_cuda and t.is_contiguous()
+    return t.data_ptr()
+
+
+# ------------------------------------------------------------------ caches
+class KVCache:
+    """cwick_hip_kv: bf16 K/V rows [capacity][n_kv_heads*head_dim] in HBM."""
+
+    def __init__(self, capacity, n_kv_heads, head_dim):
+        self.capacity, self.n_kv_heads, self.head_dim = capacity, n_kv_heads, head_dim
+        self.h = lib().cwick_hip_kv_create(capacity, n_kv_heads, head_dim)
+        if not self.h:
+            raise Declined("kv_create: " + last_error())
+
+    def write(self, pos0, k_rows, v_rows):
+        k, kp = _np(k_rows, np.uint16)
+        v, vp = _np(v_rows, np.uint16)
+        n = k.shape[0]
+        _check(lib().cwick_hip_kv_write(self.h, pos0, n, kp, vp), "kv_write")
+
+    def write_f32(self, pos0, k_rows, v_rows):
+        k, kp = _np(k_rows, np.float32)
+        v, vp = _np(v_rows, np.float32)
+        _check(lib().cwick_hip_kv_write_f32(self.h, pos0, k.shape[0], kp, vp), "kv_write_f32")
+
+    def k_dev(self):
+        return lib().cwick_hip_kv_k_dev(self.h)
+
+    def v_dev(self):
+        return lib().cwick_hip_kv_v_dev(self.h)
+
+    def free(self):
+        if self.h:
+            lib().cwick_hip_kv_free(self.h)
+            self.h = None
+
+    __del__ = free
+
+
+class LatentCache:
+    """cwick_hip_latent: FP8 rows [slots][capacity][576] + scales [..][5]."""
+
+    def __init__(self, slots, capacity):
+        self.slots, self.capacity = slots, capacity
+        self.h = lib().cwick_hip_latent_create(slots, capacity)
+        if not self.h:
+            raise Declined("latent_create: " + last_error())
+
+    def write(self, slot, pos0, rows, scales):
+        r, rp = _np(rows, np.uint8)
+        s, sp = _np(scales, np.float32)
+        assert r.shape[1] == KDIM and s.shape == (r.shape[0], NBLK)
+        _check(lib().cwick_hip_latent_write(self.h, slot, pos0, r.shape[0], rp, sp), "latent_write")
+
+    def write_f32(self, slot, pos0, rows):
+        r, rp = _np(rows, np.float32)
+        assert r.shape[1] == KDIM
+        _check(lib().cwick_hip_latent_write_f32(self.h, slot, pos0, r.shape[0], rp),
+               "latent_write_f32")
+
+    def read(self, slot, pos0, n):
+        rows = np.empty((n, KDIM), np.uint8)
+        scales = np.empty((n, NBLK), np.float32)
+        _check(lib().cwick_hip_latent_read(self.h, slot, pos0, n, rows.ctypes.data,
+                                           scales.ctypes.data), "latent_read")
+        return rows, scales
+
+    def rows_dev(self, slot=0):
+        return lib().cwick_hip_latent_rows_dev(self.h, slot)
+
+    def scales_dev(self, slot=0):
+        return lib().cwick_hip_latent_scales_dev(self.h, slot)
+
+    def free(self):
+        if self.h:
+            lib().cwick_hip_latent_free(self.h)
+            self.h = None
+
+    __del__ = free
+
+
+class IndexKeys:
+    """cwick_hip_ikeys: FP8 indexer keys [slots][capacity][128] + scale per token."""
+
+    def __init__(self, slots, capacity):
+        self.slots, self.capacity = slots, capacity
+        self.h = lib().cwick_hip_ikeys_create(slots, capacity)
+        if not self.h:
+            raise Declined("ikeys_create: " + last_error())
+
+    def write(self, slot, pos0, rows, scales):
+        r, rp = _np(rows, np.uint8)
+        s, sp = _np(scales, np.float32)
+        assert r.shape[1] == IDIM and s.size == r.shape[0]
+        _check(lib().cwick_hip_ikeys_write(self.h, slot, pos0, r.shape[0], rp, sp), "ikeys_write")
+
+    def write_f32(self, slot, pos0, rows):
+        r, rp = _np(rows, np.float32)
+        _check(lib().cwick_hip_ikeys_write_f32(self.h, slot, pos0, r.shape[0], rp),
+               "ikeys_write_f32")
+
+    def rows_dev(self, slot=0):
+        return lib().cwick_hip_ikeys_rows_dev(self.h, slot)
+
+    def scales_dev(self, slot=0):
+        return lib().cwick_hip_ikeys_scales_dev(self.h, slot)
+
+    def free(self):
+        if self.h:
+            lib().cwick_hip_ikeys_free(self.h)
+            self.h = None
+
+    __del__ = free
+
+
+# ------------------------------------------------------------------ host-pointer ops
+def gqa_decode(cache, n_keys, q, scale, raw=False):
+    q, qp = _np(q, np.uint16)
+    nh, hd = q.shape
+    out = np.empty((nh, hd), np.float32)
+    rc = lib().cwick_hip_gqa_decode(cache.h, n_keys, qp, nh, scale, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "gqa_decode")
+    return out
+
+
+def gqa_prefill(cache, pos0, q, scale, raw=False):
+    q, qp = _np(q, np.uint16)
+    n, nh, hd = q.shape
+    out = np.empty((n, nh, hd), np.float32)
+    rc = lib().cwick_hip_gqa_prefill(cache.h, pos0, n, qp, nh, scale, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "gqa_prefill")
+    return out
+
+
+def mla_decode(cache, slot, q, scale, sel=None, n_list=None, raw=False):
+    q, qp = _np(q, np.uint16)
+    nh = q.shape[0]
+    assert q.shape[1] == KDIM
+    selp = None
+    if sel is not None:
+        sel, selp = _np(sel, np.int32)
+        n_list = sel.size if n_list is None else n_list
+    out = np.empty((nh, VDIM), np.float32)
+    rc = lib().cwick_hip_mla_decode(cache.h, slot, selp, n_list, qp, nh, scale, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "mla_decode")
+    return out
+
+
+def mla_prefill_chunk(cache, slot, pos0, q, scale, raw=False):
+    q, qp = _np(q, np.uint16)
+    n, nh, kd = q.shape
+    assert kd == KDIM
+    out = np.empty((n, nh, VDIM), np.float32)
+    rc = lib().cwick_hip_mla_prefill_chunk(cache.h, slot, pos0, n, qp, nh, scale, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "mla_prefill_chunk")
+    return out
+
+
+def indexer_scores(ikeys, slot, n_keys, q_idx, w, raw=False):
+    q, qp = _np(q_idx, np.uint16)
+    w, wp = _np(w, np.float32)
+    ih = q.shape[0]
+    out = np.empty(n_keys, np.float32)
+    rc = lib().cwick_hip_indexer_scores(ikeys.h, slot, n_keys, qp, wp, ih, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "indexer_scores")
+    return out
+
+
+def topk(scores, k, raw=False):
+    s, sp = _np(scores, np.float32)
+    out = np.empty(max(k, 1), np.int32)
+    got = _i64(0)
+    rc = lib().cwick_hip_topk(sp, s.size, k, out.ctypes.data, C.byref(got))
+    if raw:
+        return rc, out[:got.value]
+    _check(rc, "topk")
+    return out[:got.value].copy()
+
+
+def dsa_decode(ikeys, latent, slot0, slot_step, n_keys, q_idx, w, topk_k, q, scale, raw=False):
+    qi, qip = _np(q_idx, np.uint16)
+    w, wp = _np(w, np.float32)
+    q, qp = _np(q, np.uint16)
+    batch, ih, _ = qi.shape
+    nh = q.shape[1]
+    out = np.empty((batch, nh, VDIM), np.float32)
+    sel = np.empty((batch, topk_k), np.int32)
+    rc = lib().cwick_hip_dsa_decode(ikeys.h, latent.h, slot0, slot_step, batch, n_keys, qip, wp,
+                                    ih, topk_k, qp, nh, scale, out.ctypes.data, sel.ctypes.data)
+    if raw:
+        return rc, out, sel
+    _check(rc, "dsa_decode")
+    return out, sel
+
+
+def e4m3_table():
+    out = np.empty(256, np.float32)
+    _check(lib().cwick_hip_e4m3_table(out.ctypes.data), "e4m3_table")
+    return out
+
+
+# ------------------------------------------------------------------ HBM-resident ops
+# Arguments are torch CUDA tensors (or raw device addresses); `stream` is a raw
+# hipStream_t address (torch.cuda.current_stream().cuda_stream) or None.
+def gqa_decode_dev(k, v, n_keys, n_kv_heads, head_dim, q, n_heads, scale, out, stream=None):
+    return _check(lib().cwick_hip_gqa_decode_dev(_dp(k), _dp(v), n_keys, n_kv_heads, head_dim,
+                                                 _dp(q), n_heads, scale, _dp(out), stream),
+                  "gqa_decode_dev")
+
+
+def gqa_prefill_dev(k, v, pos0, n, n_kv_heads, head_dim, q, n_heads, scale, out, stream=None):
+    return _check(lib().cwick_hip_gqa_prefill_dev(_dp(k), _dp(v), pos0, n, n_kv_heads, head_dim,
+                                                  _dp(q), n_heads, scale, _dp(out), stream),
+                  "gqa_prefill_dev")
+
+
+def mla_decode_dev(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list, q,
+                   n_heads, scale, out, stream=None):
+    return _check(lib().cwick_hip_mla_decode_dev(_dp(rows), _dp(scales), row_bstride,
+                                                 scale_bstride, n_rows, batch, _dp(sel), n_list,
+                                                 _dp(q), n_heads, scale, _dp(out), stream),
+                  "mla_decode_dev")
+
+
+def mla_prefill_chunk_dev(rows, scales, pos0, n, q, n_heads, scale, out, stream=None):
+    return _check(lib().cwick_hip_mla_prefill_chunk_dev(_dp(rows), _dp(scales), pos0, n, _dp(q),
+                                                        n_heads, scale, _dp(out), stream),
+                  "mla_prefill_chunk_dev")
+
+
+def indexer_scores_dev(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
+                       n_idx_heads, scores, stream=None):
+    return _check(lib().cwick_hip_indexer_scores_dev(_dp(keys), _dp(kscale), key_bstride,
+                                                     kscale_bstride, batch, n_keys, _dp(q_idx),
+                                                     _dp(w), n_idx_heads, _dp(scores), stream),
+                  "indexer_scores_dev")
+
+
+def topk_dev(scores, batch, n, k, out_idx, stream=None):
+    return _check(lib().cwick_hip_topk_dev(_dp(scores), batch, n, k, _dp(out_idx), stream),
+                  "topk_dev")
+
+
+def dsa_decode_dev(ikeys, ikscale, key_bstride, kscale_bstride, rows, scales, row_bstride,
+                   scale_bstride, batch, n_keys, q_idx, w, n_idx_heads, topk_k, q, n_heads, scale,
+                   scores_tmp, sel_out, out, stream=None):
+    return _check(lib().cwick_hip_dsa_decode_dev(
+        _dp(ikeys), _dp(ikscale), key_bstride, kscale_bstride, _dp(rows), _dp(scales),
+        row_bstride, scale_bstride, batch, n_keys, _dp(q_idx), _dp(w), n_idx_heads, topk_k,
+        _dp(q), n_heads, scale, _dp(scores_tmp), _dp(sel_out), _dp(out), stream),
+        "dsa_decode_dev")

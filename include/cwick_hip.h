@@ -1,0 +1,251 @@
+/* cwick_hip.h -- C ABI of libcwick_hip.so, the MI355X (gfx950) attention backend.
+ *
+ * The engine keeps its attention entry points (src/attention.c, src/ds_ops.c,
+ * src/q35_model.c, src/ds_model.c) and guards each hot loop with one of the
+ * calls below, the way src/h3.c:562-564 guards its CPU loop with
+ * h3_gpu_attention().  Conventions are the reference's own GPU-hook
+ * conventions (src/h3_gpu.h:19-27, src/cwick.h:480-529):
+ *
+ *   - every compute call returns 1 when the GPU produced the result and 0 when
+ *     it declined; on 0 the outputs are untouched and the caller runs its CPU
+ *     path.  A call declines on an unsupported shape, a bad argument, a
+ *     missing device or a HIP error; it never aborts and never approximates.
+ *   - cwick_hip_last_error() says why the last call on this thread declined.
+ *   - called from the request thread, one generation at a time
+ *     (src/attention.c:353-354); calls on one handle must not overlap.
+ *
+ * MI355X has its own memory, so caches live in device memory behind opaque
+ * handles that the engine fills at the sites where it writes its host caches
+ * (src/attention.c:699-709, src/q35_model.c:1649-1651, src/ds_model.c:1061-1070).
+ * Queries, index lists and outputs are host pointers, copied per call.
+ *
+ * The *_dev entry points are the same operations on memory that is already in
+ * HBM (device pointers, caller's HIP stream, no copies, no synchronisation);
+ * the host-pointer calls are thin wrappers over them.
+ *
+ * Data formats
+ *   bf16           uint16_t, the top half of an fp32 (src/util.h:55-60)
+ *   FP8            E4M3fn bytes, bias 7, no inf, 0x7F/0xFF NaN (src/tensor.c:344-368)
+ *   latent row     576 FP8 bytes = 512 "nope" dims followed by 64 rope dims;
+ *                  5 fp32 scales per row, one per 128-element block (the last
+ *                  block is the 64 rope dims); value = e4m3(byte) * scale[d/128]
+ *   indexer key    128 FP8 bytes + one fp32 scale per token
+ */
+#ifndef CWICK_HIP_H
+#define CWICK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CWICK_HIP_LATENT_KDIM 576   /* score width: nope + rope */
+#define CWICK_HIP_LATENT_VDIM 512   /* value width: nope only */
+#define CWICK_HIP_LATENT_BLOCK 128  /* elements per fp32 scale */
+#define CWICK_HIP_LATENT_NBLK 5
+#define CWICK_HIP_INDEX_DIM 128
+
+/* ---- lifecycle ------------------------------------------------------- */
+
+/* Replaces h3_gpu_ready (src/h3_gpu.h:9) / cwick_metal_backend_active
+ * (src/metal.c:120-123).  Brings device 0 up on first use.  State machine of
+ * src/h3_gpu.c:35-40: untried -> ready | unavailable (permanent).  Honours
+ * cwick_hip_force() first, then the CWICK_HIP environment variable
+ * (src/metal.c:98-105 pattern; default: on when a gfx950 device exists). */
+int cwick_hip_ready(void);
+
+/* Replaces cwick_metal_force (src/metal.c:60-79): 1 = select this backend
+ * (returns 0 on success, -1 if the device cannot be brought up), 0 = explicit
+ * CPU, every compute call declines from then on. */
+int cwick_hip_force(int on);
+
+/* Replaces h3_gpu_shutdown (src/h3_gpu.h:10): frees internal workspaces. */
+void cwick_hip_shutdown(void);
+
+/* Why the last call on this thread returned 0 / NULL ("" if it did not).
+ * Plays the part of cwick_error.message (src/cwick.h:39-59). */
+const char *cwick_hip_last_error(void);
+
+/* "gfx950 ... CUs ... GiB" into buf; returns 1, or 0 when no device is up. */
+int cwick_hip_device_info(char *buf, size_t cap);
+
+/* ---- GQA K/V cache: bf16 rows [capacity][n_kv_heads*head_dim] --------- */
+/* Device mirror of q35_model.kcache/vcache (src/q35.h:257-261), kept in the
+ * bf16 form the reference snapshots them in (src/q35_model.c:1558-1575). */
+typedef struct cwick_hip_kv cwick_hip_kv;
+cwick_hip_kv *cwick_hip_kv_create(int64_t capacity, int n_kv_heads, int head_dim);
+void cwick_hip_kv_free(cwick_hip_kv *c);
+/* Store rows pos0..pos0+n-1 (the memcpy pair of src/q35_model.c:1649-1651). */
+int cwick_hip_kv_write(cwick_hip_kv *c, int64_t pos0, int64_t n,
+                       const uint16_t *k_rows, const uint16_t *v_rows);
+/* Same from fp32 rows, narrowed on the device with round-to-nearest-even
+ * (q35_narrow_rows, src/q35_model.c:1558-1575). */
+int cwick_hip_kv_write_f32(cwick_hip_kv *c, int64_t pos0, int64_t n,
+                           const float *k_rows, const float *v_rows);
+uint16_t *cwick_hip_kv_k_dev(cwick_hip_kv *c);   /* device addresses, for */
+uint16_t *cwick_hip_kv_v_dev(cwick_hip_kv *c);   /* callers that fill in HBM */
+
+/* ---- MLA latent cache: FP8 rows + block scales ------------------------ */
+/* Device mirror of the latent cache `keys[layer][capacity][kv_lora]`
+ * (src/attention.c:78-92, src/engine.c:2894-2900) in BASELINE's FP8 format.
+ * `slots` independent sequences of `capacity` rows each (the reference's
+ * [slots][capacity][kv_lora] layout). */
+typedef struct cwick_hip_latent cwick_hip_latent;
+cwick_hip_latent *cwick_hip_latent_create(int slots, int64_t capacity);
+void cwick_hip_latent_free(cwick_hip_latent *c);
+/* Store already-quantised rows: rows [n][576] bytes, scales [n][5] fp32. */
+int cwick_hip_latent_write(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                           const uint8_t *rows, const float *scales);
+/* Store fp32 latent rows [n][576] (what src/attention.c:699-709 writes),
+ * quantised on the device: scale = amax(block)/448 (1 when the block is all
+ * zero), byte = RNE e4m3 of value/scale (src/ds_quant.c:102-128). */
+int cwick_hip_latent_write_f32(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                               const float *rows);
+/* Read rows back (for prefix snapshots, src/pfx.h:42-73). */
+int cwick_hip_latent_read(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                          uint8_t *rows, float *scales);
+uint8_t *cwick_hip_latent_rows_dev(cwick_hip_latent *c, int slot);
+float *cwick_hip_latent_scales_dev(cwick_hip_latent *c, int slot);
+
+/* ---- indexer key cache: FP8 rows [capacity][128] + scale per token ---- */
+/* Device mirror of the indexer key store (src/ds_model.c:1054-1063 idx_k,
+ * src/cwick.h:832-856 pool) in BASELINE's FP8 format. */
+typedef struct cwick_hip_ikeys cwick_hip_ikeys;
+cwick_hip_ikeys *cwick_hip_ikeys_create(int slots, int64_t capacity);
+void cwick_hip_ikeys_free(cwick_hip_ikeys *c);
+int cwick_hip_ikeys_write(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
+                          const uint8_t *rows, const float *scales);
+int cwick_hip_ikeys_write_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
+                              const float *rows);
+uint8_t *cwick_hip_ikeys_rows_dev(cwick_hip_ikeys *c, int slot);
+float *cwick_hip_ikeys_scales_dev(cwick_hip_ikeys *c, int slot);
+
+/* ---- GQA attention ---------------------------------------------------- */
+
+/* Replaces the decode branch of mixer_attn: dec_scores / dec_softmax /
+ * dec_out_slices (src/q35_model.c:1656-1701).  One query position, every
+ * head: out[h] = softmax_t(scale * q[h].K[t][h/group]) . V[.][h/group] over
+ * t in [0, n_keys).  q [n_heads][head_dim] bf16, out [n_heads][head_dim] fp32.
+ * Supported: head_dim 256 or 128, n_heads a multiple of n_kv_heads with group
+ * <= 8, 1 <= n_keys <= capacity. */
+int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q,
+                         int n_heads, float scale, float *out);
+
+/* Replaces the prefill branch of mixer_attn (src/q35_model.c:1713-1746):
+ * causal attention of n new queries at positions pos0..pos0+n-1 over cache
+ * rows 0..pos0+n-1 (which the caller has already written); query i sees keys
+ * 0..pos0+i.  q [n][n_heads][head_dim] bf16, out [n][n_heads][head_dim] fp32.
+ * Supported: head_dim 256, group = n_heads/n_kv_heads in {1,2,4,8}. */
+int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *q,
+                          int n_heads, float scale, float *out);
+
+/* ---- absorbed-latent MLA ---------------------------------------------- */
+
+/* Replaces the two reductions of mla_latent_decode (src/attention.c:749-811):
+ * scores over the latent, cwick_softmax per head, c_acc accumulation.  q is
+ * the absorbed query q_abs (after src/attention.c:741-744) as bf16
+ * [n_heads][576]; out is c_acc [n_heads][512] fp32 (before :812-815).
+ * sel == NULL: every position 0..n_list-1 (:759).  sel != NULL: n_list
+ * entries, each a row of the slot (any order, as indexer_select emits them);
+ * entries < 0 are skipped (the -1 padding of src/ds_model.c:929).
+ * Supported: 1 <= n_heads <= 128, 1 <= n_list, rows < capacity. */
+int cwick_hip_mla_decode(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
+                         const uint16_t *q, int n_heads, float scale, float *out);
+
+/* Replaces the per-token loop of cwick_attention_mla_prefill_chunk
+ * (src/attention.c:1010-1019): n queries at positions pos0..pos0+n-1, query t
+ * attends rows 0..pos0+t of the slot (npos = pos+1, :662), all of which are
+ * already written (:988-1007).  q [n][n_heads][576] bf16, out
+ * [n][n_heads][512] fp32. */
+int cwick_hip_mla_prefill_chunk(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                                const uint16_t *q, int n_heads, float scale, float *out);
+
+/* ---- DSA: lightning indexer, top-k, sparse MLA ------------------------- */
+
+/* Replaces the score loop of indexer_select (src/attention.c:573-582) and of
+ * ds_indexer (src/ds_model.c:1108-1121): scores[t] = sum_h relu(q_h.k_t) * w[h]
+ * for t in [0, n_keys).  q_idx [n_idx_heads][128] bf16, w [n_idx_heads] fp32
+ * (already folded with 1/sqrt(hd*ih), :564-565).  The summation order is
+ * fixed and documented beside the kernel, so the result is bit-identical to
+ * the CPU oracle that follows the same order.  n_idx_heads <= 64. */
+int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys,
+                             const uint16_t *q_idx, const float *w, int n_idx_heads,
+                             float *scores);
+
+/* Replaces ds_topk_scores (src/ds_ops.c:310-338, contract src/ds_ops.h:110-112)
+ * and the threshold selector of src/attention.c:585-598: the k best of n
+ * scores by (score descending, index ascending), written in ascending index
+ * order.  -0.0 == +0.0; NaN ranks below -inf.  *n_out = min(k, n).
+ * n <= 2^24, k <= 65536. */
+int cwick_hip_topk(const float *scores, int64_t n, int64_t k, int32_t *out_idx,
+                   int64_t *n_out);
+
+/* Replaces the indexer -> top-k -> sparse attention chain of a DSA decode
+ * step (src/ds_model.c:1081-1164 + :968-995; src/attention.c:716-811) for a
+ * batch of independent queries: query b reads slot slot0 + b*slot_step of
+ * both caches (slot_step 0 = one shared context).
+ * q_idx [batch][n_idx_heads][128] bf16, w [batch][n_idx_heads], q
+ * [batch][n_heads][576] bf16, out [batch][n_heads][512] fp32; sel_out, when
+ * not NULL, receives the selected rows [batch][topk] (ascending, -1 padded
+ * when n_keys < topk). */
+int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, int slot_step,
+                         int batch, int64_t n_keys, const uint16_t *q_idx, const float *w,
+                         int n_idx_heads, int64_t topk, const uint16_t *q, int n_heads,
+                         float scale, float *out, int32_t *sel_out);
+
+/* ---- the same operations on HBM-resident operands ---------------------- */
+/* All pointers are device pointers; `stream` is a hipStream_t (NULL = the
+ * null stream).  Kernels are enqueued, nothing is copied or waited for.
+ * Scratch for split-K partials comes from a grow-only per-device workspace
+ * inside the library. */
+
+int cwick_hip_gqa_decode_dev(const uint16_t *k, const uint16_t *v, int64_t n_keys,
+                             int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
+                             float scale, float *out, void *stream);
+
+int cwick_hip_gqa_prefill_dev(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
+                              int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
+                              float scale, float *out, void *stream);
+
+/* batch queries; query b uses rows + b*row_batch_stride (bytes) and
+ * scales + b*scale_batch_stride (floats), each holding n_rows valid rows;
+ * sel [batch][n_list] or NULL.  sel entries outside [0, n_rows) are skipped. */
+int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales,
+                             int64_t row_batch_stride, int64_t scale_batch_stride,
+                             int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
+                             const uint16_t *q, int n_heads, float scale, float *out,
+                             void *stream);
+
+int cwick_hip_mla_prefill_chunk_dev(const uint8_t *rows, const float *scales, int64_t pos0,
+                                    int64_t n, const uint16_t *q, int n_heads, float scale,
+                                    float *out, void *stream);
+
+int cwick_hip_indexer_scores_dev(const uint8_t *keys, const float *kscale,
+                                 int64_t key_batch_stride, int64_t kscale_batch_stride,
+                                 int batch, int64_t n_keys, const uint16_t *q_idx,
+                                 const float *w, int n_idx_heads, float *scores,
+                                 void *stream);
+
+/* scores [batch][n], out_idx [batch][k] (rows padded with -1 past min(k,n)). */
+int cwick_hip_topk_dev(const float *scores, int batch, int64_t n, int64_t k,
+                       int32_t *out_idx, void *stream);
+
+int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale,
+                             int64_t key_batch_stride, int64_t kscale_batch_stride,
+                             const uint8_t *rows, const float *scales,
+                             int64_t row_batch_stride, int64_t scale_batch_stride,
+                             int batch, int64_t n_keys, const uint16_t *q_idx, const float *w,
+                             int n_idx_heads, int64_t topk, const uint16_t *q, int n_heads,
+                             float scale, float *scores_tmp, int32_t *sel_out, float *out,
+                             void *stream);
+
+/* Device-side codec check used by the parity tests: decodes all 256 E4M3
+ * bytes with the conversion instruction the kernels use into out256 (host). */
+int cwick_hip_e4m3_table(float *out256);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CWICK_HIP_H */

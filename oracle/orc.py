@@ -1,0 +1,258 @@
+"""ctypes front end of the CPU oracle (oracle/cwick_oracle.c) and of oracle/_ref.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg as the checker / reported CPU baseline.  The shipped
+package (cwick_amd) never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libcwick_oracle.so")
+_REF = os.path.join(_HERE, "_ref", "libcwick_ref.so")
+
+KDIM, VDIM, BLOCK = 576, 512, 128
+
+
+def build(force=False):
+    """Compile the restatement (and _ref when the reference tree is present)."""
+    if force or not os.path.exists(_LIB):
+        subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []))
+    return _LIB
+
+
+_lib = None
+_ref = None
+
+
+def _p(a, ct):
+    return a.ctypes.data_as(C.POINTER(ct))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            build()
+        L = C.CDLL(_LIB)
+        L.orc_bf16_to_f32.restype = C.c_float
+        L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_bf16_rne.restype = C.c_uint16
+        L.orc_f32_to_bf16_rne.argtypes = [C.c_float]
+        L.orc_f32_to_bf16_cwick.restype = C.c_uint16
+        L.orc_f32_to_bf16_cwick.argtypes = [C.c_float]
+        L.orc_bf16_round.restype = C.c_float
+        L.orc_bf16_round.argtypes = [C.c_float]
+        L.orc_e4m3_to_f32.restype = C.c_float
+        L.orc_e4m3_to_f32.argtypes = [C.c_uint8]
+        L.orc_f32_to_e4m3.restype = C.c_uint8
+        L.orc_f32_to_e4m3.argtypes = [C.c_float]
+        L.orc_f32_to_e4m3_rne.restype = C.c_uint8
+        L.orc_f32_to_e4m3_rne.argtypes = [C.c_float]
+        L.orc_dot_f32.restype = C.c_float
+        L.orc_topk_contract.restype = C.c_int64
+        L.orc_topk_quickselect.restype = C.c_int64
+        L.orc_topk_heap.restype = C.c_int
+        L.orc_topk_order_key.restype = C.c_uint32
+        L.orc_topk_order_key.argtypes = [C.c_float]
+        L.orc_now_ns.restype = C.c_int64
+        L.orc_max_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def ref():
+    """The reference's own object code (oracle/_ref), or None if it was not built."""
+    global _ref
+    if _ref is None and os.path.exists(_REF):
+        R = C.CDLL(_REF)
+        R.cwick_fp8_e4m3_to_f32.restype = C.c_float
+        R.cwick_fp8_e4m3_to_f32.argtypes = [C.c_uint8]
+        R.cwick_bf16_to_f32.restype = C.c_float
+        R.cwick_bf16_to_f32.argtypes = [C.c_uint16]
+        R.cwick_f32_to_bf16.restype = C.c_uint16
+        R.cwick_f32_to_bf16.argtypes = [C.c_float]
+        R.ds_bf16_round.restype = C.c_float
+        R.ds_bf16_round.argtypes = [C.c_float]
+        R.ds_topk_scores.restype = C.c_int
+        _ref = R
+    return _ref
+
+
+def max_threads():
+    return int(lib().orc_max_threads())
+
+
+# ---------------------------------------------------------------- codecs
+def e4m3_lut():
+    out = np.empty(256, np.float32)
+    lib().orc_e4m3_lut(_p(out, C.c_float))
+    return out
+
+
+def quantize_rows_e4m3(x, block):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    nb = (cols + block - 1) // block
+    q = np.empty((rows, cols), np.uint8)
+    s = np.empty((rows, nb), np.float32)
+    lib().orc_quantize_rows_e4m3(_p(x, C.c_float), C.c_int64(rows), C.c_int64(cols),
+                                 C.c_int64(block), _p(q, C.c_uint8), _p(s, C.c_float))
+    return q, s
+
+
+def softmax(x):
+    x = np.array(x, np.float32, copy=True)
+    lib().orc_softmax(_p(x, C.c_float), C.c_int64(x.size))
+    return x
+
+
+def dot_f32(a, b):
+    a = np.ascontiguousarray(a, np.float32)
+    b = np.ascontiguousarray(b, np.float32)
+    return float(lib().orc_dot_f32(_p(a, C.c_float), _p(b, C.c_float), C.c_int64(a.size)))
+
+
+# ---------------------------------------------------------------- attention
+def gqa_decode(q, k, v, scale, nslice=16, nthreads=1):
+    """q [nh,hd] u16, k/v [keys,nkv,hd] u16 -> [nh,hd] f32."""
+    q = np.ascontiguousarray(q, np.uint16)
+    k = np.ascontiguousarray(k, np.uint16)
+    v = np.ascontiguousarray(v, np.uint16)
+    nh, hd = q.shape
+    keys, nkv, _ = k.shape
+    out = np.empty((nh, hd), np.float32)
+    lib().orc_gqa_decode(_p(q, C.c_uint16), _p(k, C.c_uint16), _p(v, C.c_uint16),
+                         C.c_int64(keys), nh, nkv, hd, C.c_float(scale), nslice, nthreads,
+                         _p(out, C.c_float))
+    return out
+
+
+def gqa_prefill(q, k, v, pos0, scale, tile_q=128, tiles=(0, 0, 1), nthreads=1, out=None):
+    """q [n,nh,hd] u16, k/v [pos0+n,nkv,hd] u16 -> [n,nh,hd] f32 (causal)."""
+    q = np.ascontiguousarray(q, np.uint16)
+    k = np.ascontiguousarray(k, np.uint16)
+    v = np.ascontiguousarray(v, np.uint16)
+    n, nh, hd = q.shape
+    nkv = k.shape[1]
+    assert k.shape[0] >= pos0 + n
+    if out is None:
+        out = np.zeros((n, nh, hd), np.float32)
+    lib().orc_gqa_prefill(_p(q, C.c_uint16), _p(k, C.c_uint16), _p(v, C.c_uint16),
+                          C.c_int64(pos0), C.c_int64(n), nh, nkv, hd, C.c_float(scale),
+                          tile_q, C.c_int64(tiles[0]), C.c_int64(tiles[1]), C.c_int64(tiles[2]),
+                          nthreads, _p(out, C.c_float))
+    return out
+
+
+def mla_decode(q, lat, scales, scale, sel=None, nlist=None, nthreads=1,
+               kdim=KDIM, vdim=VDIM, block=BLOCK):
+    """q [nh,kdim] u16, lat [cap,kdim] u8, scales [cap,nblk] f32 -> [nh,vdim] f32."""
+    q = np.ascontiguousarray(q, np.uint16)
+    lat = np.ascontiguousarray(lat, np.uint8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    nh = q.shape[0]
+    if sel is not None:
+        sel = np.ascontiguousarray(sel, np.int32)
+        nlist = sel.size if nlist is None else nlist
+        selp = _p(sel, C.c_int32)
+    else:
+        nlist = lat.shape[0] if nlist is None else nlist
+        selp = None
+    out = np.empty((nh, vdim), np.float32)
+    lib().orc_mla_decode(_p(q, C.c_uint16), _p(lat, C.c_uint8), _p(scales, C.c_float),
+                         C.c_int64(kdim), C.c_int64(vdim), C.c_int64(block), selp,
+                         C.c_int64(nlist), nh, C.c_float(scale), nthreads, _p(out, C.c_float))
+    return out
+
+
+def mla_decode_f32(q_abs, lat, scale, sel=None, nlist=None):
+    q_abs = np.ascontiguousarray(q_abs, np.float32)
+    lat = np.ascontiguousarray(lat, np.float32)
+    nh, dim = q_abs.shape
+    if sel is not None:
+        sel = np.ascontiguousarray(sel, np.int64)
+        nlist = sel.size
+        selp = _p(sel, C.c_int64)
+    else:
+        nlist = lat.shape[0] if nlist is None else nlist
+        selp = None
+    out = np.empty((nh, dim), np.float32)
+    lib().orc_mla_decode_f32(_p(q_abs, C.c_float), _p(lat, C.c_float), C.c_int64(dim), selp,
+                             C.c_int64(nlist), nh, C.c_float(scale), _p(out, C.c_float))
+    return out
+
+
+def mla_prefill_chunk(q, lat, scales, pos0, scale, queries=(0, 0, 1), nthreads=1, out=None,
+                      kdim=KDIM, vdim=VDIM, block=BLOCK):
+    """q [n,nh,kdim] u16 -> [n,nh,vdim] f32; causal over positions 0..pos0+t."""
+    q = np.ascontiguousarray(q, np.uint16)
+    lat = np.ascontiguousarray(lat, np.uint8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    n, nh, _ = q.shape
+    assert lat.shape[0] >= pos0 + n
+    if out is None:
+        out = np.zeros((n, nh, vdim), np.float32)
+    lib().orc_mla_prefill_chunk(_p(q, C.c_uint16), _p(lat, C.c_uint8), _p(scales, C.c_float),
+                                C.c_int64(kdim), C.c_int64(vdim), C.c_int64(block),
+                                C.c_int64(pos0), C.c_int64(n), nh, C.c_float(scale),
+                                C.c_int64(queries[0]), C.c_int64(queries[1]),
+                                C.c_int64(queries[2]), nthreads, _p(out, C.c_float))
+    return out
+
+
+def indexer_scores(q, w, keys, kscale, n=None, nthreads=1):
+    """q [ih,hd] u16, w [ih] f32, keys [n,hd] u8, kscale [n] f32 -> [n] f32."""
+    q = np.ascontiguousarray(q, np.uint16)
+    w = np.ascontiguousarray(w, np.float32)
+    keys = np.ascontiguousarray(keys, np.uint8)
+    kscale = np.ascontiguousarray(kscale, np.float32)
+    ih, hd = q.shape
+    n = keys.shape[0] if n is None else n
+    sc = np.empty(n, np.float32)
+    lib().orc_indexer_scores(_p(q, C.c_uint16), _p(w, C.c_float), _p(keys, C.c_uint8),
+                             _p(kscale, C.c_float), C.c_int64(n), ih, hd, nthreads,
+                             _p(sc, C.c_float))
+    return sc
+
+
+def topk_contract(sc, k):
+    sc = np.ascontiguousarray(sc, np.float32)
+    out = np.empty(max(min(k, sc.size), 1), np.int32)
+    got = lib().orc_topk_contract(_p(sc, C.c_float), C.c_int64(sc.size), C.c_int64(k),
+                                  _p(out, C.c_int32))
+    return out[:got].copy()
+
+
+def topk_heap(sc, k):
+    sc = np.ascontiguousarray(sc, np.float32)
+    out = np.empty(max(k, 1), np.int32)
+    got = lib().orc_topk_heap(_p(sc, C.c_float), int(sc.size), int(k), _p(out, C.c_int32))
+    return out[:got].copy()
+
+
+def topk_quickselect(sc, want):
+    sc = np.ascontiguousarray(sc, np.float32)
+    out = np.empty(sc.size, np.int32)
+    got = lib().orc_topk_quickselect(_p(sc, C.c_float), C.c_int64(sc.size), C.c_int64(want),
+                                     _p(out, C.c_int32))
+    return out[:got].copy()
+
+
+def ref_topk_scores(sc, k):
+    """ds_topk_scores as compiled from the reference (src/ds_ops.c:310-338)."""
+    R = ref()
+    sc = np.ascontiguousarray(sc, np.float32)
+    out = np.empty(max(k, 1), np.int32)
+    heap = np.empty(max(k, 1), np.float32)
+    hidx = np.empty(max(k, 1), np.int32)
+    got = R.ds_topk_scores(_p(sc, C.c_float), int(sc.size), int(k), _p(out, C.c_int32),
+                           _p(heap, C.c_float), _p(hidx, C.c_int32))
+    return out[:got].copy()
+
+
+def now_ns():
+    return int(lib().orc_now_ns())

@@ -1,0 +1,195 @@
+"""GPU parity: libcwick_hip.so through its C ABI against the CPU oracle on the
+same seeded inputs.  Bit-exact for codecs, indexer scores and top-k indices;
+max-abs 2e-3 / rel 1e-2 for attention outputs (bf16/fp8 in, fp32 accumulate)."""
+import numpy as np
+import pytest
+
+from cwick_amd import synth
+from tests.conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------ codecs
+def test_e4m3_hardware_decode_matches_table(hip, orc):
+    say("[case] e4m3 table")
+    got = hip.e4m3_table()
+    ref = orc.e4m3_lut()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    assert np.array_equal(got[ok].view(np.uint32), ref[ok].view(np.uint32))
+
+
+def test_latent_quantise_on_append_bit_exact(hip, orc):
+    say("[case] latent write_f32")
+    g = synth.rng(11)
+    x = g.standard_normal((300, synth.KDIM), dtype=np.float32)
+    x[5] = 0.0
+    x[6, :128] = 0.0
+    x[7] *= 1e-6
+    x[8] *= 1e4
+    c = hip.LatentCache(2, 512)
+    c.write_f32(1, 100, x)
+    rows, scales = c.read(1, 100, 300)
+    rq, rs = orc.quantize_rows_e4m3(x, 128)
+    assert np.array_equal(scales.view(np.uint32), rs.view(np.uint32))
+    assert np.array_equal(rows, rq)
+    nq, ns = synth.quantize_rows(x, 128)
+    assert np.array_equal(nq, rq) and np.array_equal(ns.view(np.uint32), rs.view(np.uint32))
+    c.free()
+
+
+# ------------------------------------------------------------------ GQA decode
+@pytest.mark.parametrize("n_keys,nh,nkv,hd", [
+    (4096, 16, 4, 256),      # BASELINE config 1
+    (1, 16, 4, 256),
+    (63, 16, 4, 256),
+    (1000, 8, 8, 128),
+    (777, 32, 4, 128),
+    (513, 8, 4, 256),
+])
+def test_gqa_decode(hip, orc, n_keys, nh, nkv, hd):
+    say("[case] gqa_decode", n_keys, nh, nkv, hd)
+    c = synth.cfg1_gqa_decode(n_keys, nh, nkv, hd, seed=100 + n_keys)
+    cache = hip.KVCache(n_keys + 7, nkv, hd)
+    cache.write(0, c["k"].reshape(n_keys, -1), c["v"].reshape(n_keys, -1))
+    got = hip.gqa_decode(cache, n_keys, c["q"], c["scale"])
+    ref = orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"])
+    assert_close(got, ref, "gqa_decode %d keys %d/%d/%d" % (n_keys, nh, nkv, hd))
+    cache.free()
+
+
+# ------------------------------------------------------------------ MLA decode
+@pytest.mark.parametrize("n_keys,nh", [
+    (32768, 128),            # BASELINE config 3
+    (1, 128),
+    (65, 128),
+    (2051, 64),              # the reference's released geometry (src/attention.c:341-343)
+    (700, 16),
+    (300, 40),
+])
+def test_mla_decode_dense(hip, orc, n_keys, nh):
+    say("[case] mla_decode dense", n_keys, nh)
+    c = synth.cfg3_mla_decode(n_keys, nh, seed=300 + n_keys)
+    cache = hip.LatentCache(1, n_keys)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_decode(cache, 0, c["q"], c["scale"], n_list=n_keys)
+    ref = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=0)
+    assert_close(got, ref, "mla_decode dense %d keys %d heads" % (n_keys, nh))
+    cache.free()
+
+
+def test_mla_decode_sel(hip, orc):
+    say("[case] mla_decode sel")
+    n_rows, nh = 5000, 128
+    c = synth.cfg3_mla_decode(n_rows, nh, seed=77)
+    g = synth.rng(78)
+    sel = g.permutation(n_rows)[:2048].astype(np.int32)     # any order, as the selector emits
+    sel[[3, 500, 2047]] = -1                                 # -1 padding is skipped
+    cache = hip.LatentCache(2, n_rows)
+    cache.write(1, 0, c["rows"], c["scales"])
+    got = hip.mla_decode(cache, 1, c["q"], c["scale"], sel=sel)
+    ref = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=sel, nthreads=0)
+    assert_close(got, ref, "mla_decode sel 2048 of 5000")
+    # order of the list does not matter beyond rounding
+    got2 = hip.mla_decode(cache, 1, c["q"], c["scale"], sel=np.sort(sel))
+    assert_close(got2, ref, "mla_decode sel sorted")
+    # a list entry outside the cache is refused on the host, outputs untouched
+    bad = sel.copy()
+    bad[0] = n_rows
+    rc, _ = hip.mla_decode(cache, 1, c["q"], c["scale"], sel=bad, raw=True)
+    assert rc == 0 and "outside" in hip.last_error()
+    cache.free()
+
+
+# ------------------------------------------------------------------ MLA prefill
+@pytest.mark.parametrize("pos0,n,nh", [(0, 70, 128), (200, 33, 64), (1000, 5, 16)])
+def test_mla_prefill_chunk(hip, orc, pos0, n, nh):
+    say("[case] mla_prefill_chunk", pos0, n, nh)
+    c = synth.cfg4_mla_prefill(n, pos0, nh, seed=400 + n)
+    cache = hip.LatentCache(1, pos0 + n)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_prefill_chunk(cache, 0, pos0, c["q"], c["scale"])
+    ref = orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"], nthreads=0)
+    assert_close(got, ref, "mla_prefill pos0 %d n %d heads %d" % (pos0, n, nh))
+    cache.free()
+
+
+# ------------------------------------------------------------------ indexer + top-k
+@pytest.mark.parametrize("n_keys,ih", [(65536, 64), (1, 64), (1000, 32), (257, 7)])
+def test_indexer_scores_bit_exact(hip, orc, n_keys, ih):
+    say("[case] indexer_scores", n_keys, ih)
+    g = synth.rng(500 + n_keys)
+    keys, ks = synth.index_keys(g, n_keys)
+    q = synth.normal_bf16(g, (ih, synth.IDIM))
+    w = (g.standard_normal(ih, dtype=np.float32) / np.float32(np.sqrt(128.0 * ih))).astype(np.float32)
+    cache = hip.IndexKeys(1, n_keys)
+    cache.write(0, 0, keys, ks)
+    got = hip.indexer_scores(cache, 0, n_keys, q, w)
+    ref = orc.indexer_scores(q, w, keys, ks, nthreads=0)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "indexer scores differ in %d of %d places" % ((got != ref).sum(), n_keys)
+    cache.free()
+
+
+TOPK_KNOWN = [
+    ([5, 5, 7], 2, [0, 2]),                      # ds_topk_scores returns {1,2} here
+    ([3, 9, 3, 3, 8, 3], 4, [0, 1, 2, 4]),       # ... and {1,2,3,4} here
+    ([1, 1, 1, 1, 1], 3, [0, 1, 2]),
+    ([2, 1], 5, [0, 1]),
+    ([0.0, -0.0, 1.0, -0.0], 3, [0, 1, 2]),
+    ([-np.inf, 1, -np.inf, 2], 3, [0, 1, 3]),
+]
+
+
+@pytest.mark.parametrize("sc,k,want", TOPK_KNOWN)
+def test_topk_known_answers(hip, orc, sc, k, want):
+    say("[case] topk known", sc, k)
+    sc = np.array(sc, np.float32)
+    assert list(orc.topk_contract(sc, k)) == want
+    assert list(hip.topk(sc, k)) == want
+
+
+@pytest.mark.parametrize("n,k,kind", [
+    (65536, 2048, "normal"), (65536, 2048, "ties"), (65536, 2048, "const"),
+    (100000, 512, "normal"), (5000, 5000, "normal"), (3000, 4096, "ties"),
+    (1 << 20, 2048, "ties"), (777, 1, "normal"), (4097, 2048, "inf"),
+])
+def test_topk_bit_exact(hip, orc, n, k, kind):
+    say("[case] topk", n, k, kind)
+    g = synth.rng(600 + n + k)
+    if kind == "normal":
+        sc = g.standard_normal(n, dtype=np.float32)
+    elif kind == "ties":
+        sc = g.integers(-20, 20, n).astype(np.float32) * np.float32(0.25)
+    elif kind == "const":
+        sc = np.full(n, 1.5, np.float32)
+    else:
+        sc = g.standard_normal(n, dtype=np.float32)
+        sc[g.random(n) < 0.7] = -np.inf
+    got = hip.topk(sc, k)
+    ref = orc.topk_contract(sc, k)
+    assert np.array_equal(got, ref)
+
+
+def test_dsa_decode_small(hip, orc):
+    say("[case] dsa_decode small")
+    c = synth.cfg5_dsa(n_keys=3000, batch=3, ih=64, topk=256, nh=128, seed=909)
+    ik = hip.IndexKeys(3, 3000)
+    lat = hip.LatentCache(3, 3000)
+    for b in range(3):
+        ik.write(b, 0, c["ikeys"][b], c["ikscale"][b])
+        lat.write(b, 0, c["rows"][b], c["scales"][b])
+    out, sel = hip.dsa_decode(ik, lat, 0, 1, 3000, c["q_idx"], c["w"], 256, c["q"], c["scale"])
+    for b in range(3):
+        sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], c["ikeys"][b], c["ikscale"][b], nthreads=0)
+        rsel = orc.topk_contract(sc, 256)
+        assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
+        ref = orc.mla_decode(c["q"][b], c["rows"][b], c["scales"][b], c["scale"], sel=rsel, nthreads=0)
+        assert_close(out[b], ref, "dsa_decode query %d" % b)
+    ik.free()
+    lat.free()

@@ -1,0 +1,188 @@
+"""Pins the attention functions of the CPU oracle with mathematics that a plausible
+mistake (a dropped term, a wrong sign or index, a transposed operand, a wrong head
+map, an off-by-one in the causal limit) would break: brute force in double precision
+written independently in numpy, and the identities the reference itself relies on."""
+import numpy as np
+import pytest
+
+from cwick_amd import synth
+
+
+def f32(b):
+    return synth.bf16_to_f32(b).astype(np.float64)
+
+
+def softmax64(s, axis=-1):
+    s = s - s.max(axis=axis, keepdims=True)
+    e = np.exp(s)
+    return e / e.sum(axis=axis, keepdims=True)
+
+
+def dequant(rows, scales, lut):
+    return lut[rows].astype(np.float64) * np.repeat(scales.astype(np.float64), 128, axis=1)[:, :rows.shape[1]]
+
+
+# ------------------------------------------------------------------ GQA
+def brute_gqa(q, k, v, scale, limit=None):
+    """q [nh,hd], k/v [keys,nkv,hd] float64; head h reads kv head h // group."""
+    nh, hd = q.shape
+    keys, nkv, _ = k.shape
+    group = nh // nkv
+    out = np.zeros((nh, hd))
+    n = keys if limit is None else limit
+    for h in range(nh):
+        g = h // group
+        p = softmax64(scale * (k[:n, g] @ q[h]))
+        out[h] = p @ v[:n, g]
+    return out
+
+
+@pytest.mark.parametrize("keys,nh,nkv,hd", [(300, 16, 4, 256), (1, 4, 4, 64), (97, 8, 2, 128)])
+def test_gqa_decode_vs_brute_force(orc, keys, nh, nkv, hd):
+    c = synth.cfg1_gqa_decode(keys, nh, nkv, hd, seed=keys)
+    got = orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"])
+    want = brute_gqa(f32(c["q"]), f32(c["k"]), f32(c["v"]), c["scale"])
+    assert np.abs(got - want).max() < 2e-5
+    # slicing and threading only reorder the fp32 sums
+    for ns, nt in [(1, 1), (7, 3), (16, 0)]:
+        assert np.abs(orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"], ns, nt) - want).max() < 2e-5
+
+
+def test_gqa_decode_attnbench_inputs(orc):
+    """The deterministic fixture of tools/attnbench.c:142-149."""
+    keys, nkv, hd, nh = 257, 4, 256, 16
+    i = np.arange(keys * nkv * hd, dtype=np.int64)
+    kf = ((i * 37) % 101 - 50).astype(np.float32) * np.float32(0.02)
+    k = (kf.view(np.uint32) >> 16).astype(np.uint16).reshape(keys, nkv, hd)      # truncation, as there
+    v = synth.f32_to_bf16(((i * 13) % 89 - 44).astype(np.float32) * np.float32(0.01)).reshape(keys, nkv, hd)
+    j = np.arange(nh * hd, dtype=np.int64)
+    q = synth.f32_to_bf16(((j * 17) % 67 - 33).astype(np.float32) * np.float32(0.03)).reshape(nh, hd)
+    got = orc.gqa_decode(q, k, v, 0.0625)
+    assert np.abs(got - brute_gqa(f32(q), f32(k), f32(v), 0.0625)).max() < 2e-5
+
+
+@pytest.mark.parametrize("pos0,n", [(0, 150), (37, 40)])
+def test_gqa_prefill_vs_brute_force_and_decode(orc, pos0, n):
+    nh, nkv, hd = 8, 2, 64
+    c = synth.cfg2_gqa_prefill(n, nh, nkv, hd, pos0, seed=n)
+    got = orc.gqa_prefill(c["q"], c["k"], c["v"], pos0, c["scale"], tile_q=64)
+    q, k, v = f32(c["q"]), f32(c["k"]), f32(c["v"])
+    for t in range(n):
+        want = brute_gqa(q[t], k, v, c["scale"], limit=pos0 + t + 1)
+        assert np.abs(got[t] - want).max() < 2e-5, t
+    # prefill row t == decode at position pos0+t (the reference runs either, n == 1 or not)
+    for t in (0, n // 2, n - 1):
+        dec = orc.gqa_decode(c["q"][t], c["k"][:pos0 + t + 1], c["v"][:pos0 + t + 1], c["scale"])
+        assert np.abs(got[t] - dec).max() < 2e-5
+    # the -1e30 rectangle equals the triangle: tile size must not matter
+    other = orc.gqa_prefill(c["q"], c["k"], c["v"], pos0, c["scale"], tile_q=7, nthreads=0)
+    assert np.abs(got - other).max() < 2e-5
+    # tile sub-sampling touches only the chosen tiles
+    part = orc.gqa_prefill(c["q"], c["k"], c["v"], pos0, c["scale"], tile_q=16, tiles=(1, 0, 3))
+    for tile in range((n + 15) // 16):
+        rows = slice(tile * 16, min(n, tile * 16 + 16))
+        if tile >= 1 and (tile - 1) % 3 == 0:
+            assert np.abs(part[rows] - got[rows]).max() < 2e-5
+        else:
+            assert not part[rows].any()
+
+
+# ------------------------------------------------------------------ MLA
+def brute_mla(q, lat, scale, sel=None):
+    """q [nh,576] f64, lat [rows,576] f64: K = all 576 dims, V = first 512."""
+    rows = lat if sel is None else lat[[t for t in sel if t >= 0]]
+    p = softmax64(scale * (q @ rows.T), axis=1)
+    return p @ rows[:, :512]
+
+
+@pytest.mark.parametrize("n,nh", [(1, 4), (200, 16), (1000, 128)])
+def test_mla_decode_vs_brute_force(orc, n, nh):
+    c = synth.cfg3_mla_decode(n, nh, seed=n)
+    lut = orc.e4m3_lut()
+    lat = dequant(c["rows"], c["scales"], lut)
+    want = brute_mla(f32(c["q"]), lat, c["scale"])
+    got = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"])
+    assert np.abs(got - want).max() < 1e-5
+    assert np.abs(orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=0) - want).max() < 1e-5
+    # dense == sel = 0..n-1, bit for bit (same order of operations)
+    same = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=np.arange(n, dtype=np.int32))
+    assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
+
+
+def test_mla_decode_sel_gather_and_padding(orc):
+    n, nh = 700, 32
+    c = synth.cfg3_mla_decode(n, nh, seed=5)
+    lat = dequant(c["rows"], c["scales"], orc.e4m3_lut())
+    g = synth.rng(6)
+    sel = g.permutation(n)[:256].astype(np.int32)
+    want = brute_mla(f32(c["q"]), lat, c["scale"], sel)
+    got = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=sel)
+    assert np.abs(got - want).max() < 1e-5
+    # softmax is order-free: a permuted list changes only rounding
+    assert np.abs(orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=np.sort(sel)) - want).max() < 1e-5
+    # -1 slots contribute nothing (src/ds_model.c:929/:940/:950)
+    padded = np.concatenate([sel[:100], [-1, -1], sel[100:], [-1]]).astype(np.int32)
+    assert np.abs(orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=padded) - want).max() < 1e-5
+    assert not orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"],
+                              sel=np.full(4, -1, np.int32)).any()
+
+
+def test_mla_absorption_identity(orc):
+    """The check the reference runs on itself (src/attention.c:838-893): the absorbed
+    form over the latent equals classic attention over k_t = W_k c_t, v_t = W_v c_t."""
+    g = synth.rng(7)
+    nh, dim, nope, vdim, n = 4, 32, 16, 24, 50
+    lat = g.standard_normal((n, dim)).astype(np.float32)
+    q = g.standard_normal((nh, nope)).astype(np.float32)
+    wk = g.standard_normal((nh, nope, dim)).astype(np.float32)
+    wv = g.standard_normal((nh, vdim, dim)).astype(np.float32)
+    scale = 1.0 / np.sqrt(nope)
+    q_abs = np.einsum("hi,hic->hc", q, wk).astype(np.float32)             # :741-744
+    c_acc = orc.mla_decode_f32(q_abs, lat, scale)
+    absorbed = np.einsum("hvc,hc->hv", wv.astype(np.float64), c_acc.astype(np.float64))   # :812-815
+    for h in range(nh):
+        k = lat.astype(np.float64) @ wk[h].astype(np.float64).T
+        v = lat.astype(np.float64) @ wv[h].astype(np.float64).T
+        p = softmax64(scale * (k @ q[h].astype(np.float64)))
+        assert np.abs(absorbed[h] - p @ v).max() < 1e-4
+
+
+def test_mla_prefill_is_a_loop_of_decodes(orc):
+    pos0, n, nh = 90, 20, 16
+    c = synth.cfg4_mla_prefill(n, pos0, nh, seed=8)
+    got = orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"])
+    lat = dequant(c["rows"], c["scales"], orc.e4m3_lut())
+    for t in range(n):
+        dec = orc.mla_decode(c["q"][t], c["rows"], c["scales"], c["scale"], nlist=pos0 + t + 1)
+        assert np.array_equal(got[t].view(np.uint32), dec.view(np.uint32))
+        want = brute_mla(f32(c["q"][t]), lat[:pos0 + t + 1], c["scale"])
+        assert np.abs(got[t] - want).max() < 1e-5
+    part = orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"], queries=(2, 0, 5))
+    for t in range(n):
+        if t >= 2 and (t - 2) % 5 == 0:
+            assert np.array_equal(part[t], got[t])
+        else:
+            assert not part[t].any()
+
+
+# ------------------------------------------------------------------ indexer
+def test_indexer_scores_vs_brute_force(orc):
+    g = synth.rng(9)
+    n, ih = 500, 64
+    keys, ks = synth.index_keys(g, n)
+    q = synth.normal_bf16(g, (ih, 128))
+    w = (g.standard_normal(ih) / np.sqrt(128.0 * ih)).astype(np.float32)
+    got = orc.indexer_scores(q, w, keys, ks)
+    lut = orc.e4m3_lut().astype(np.float64)
+    d = (lut[keys] * ks[:, None].astype(np.float64)) @ f32(q).T           # [n, ih]
+    want = (np.maximum(d, 0.0) * w.astype(np.float64)).sum(axis=1)        # ReLU BEFORE the weight
+    assert np.abs(got - want).max() < 1e-5
+    wrong = np.maximum(d * w.astype(np.float64), 0.0).sum(axis=1)         # ReLU after: a different function
+    assert np.abs(got - wrong).max() > 1e-2
+    # threads do not change a single bit (each key's sum is private)
+    assert np.array_equal(got.view(np.uint32), orc.indexer_scores(q, w, keys, ks, nthreads=0).view(np.uint32))
+    # a positive per-token scale commutes with the ReLU: scaling a key's scale by 4
+    # (exact in fp32) scales its score by 4
+    ks2 = ks.copy()
+    ks2[10] *= np.float32(4.0)
+    assert orc.indexer_scores(q, w, keys, ks2)[10] == np.float32(4.0) * got[10]
