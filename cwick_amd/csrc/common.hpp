@@ -38,6 +38,16 @@ void *workspace(hipStream_t s, size_t bytes);
 // operands by the host-pointer entry points).
 void *staging(hipStream_t s, size_t bytes);
 
+// Phase timer: brackets the launches made while it is alive with two events on
+// `s` when profiling is enabled; does nothing (and records nothing) otherwise.
+struct ProfScope {
+    ProfScope(int which, hipStream_t s);
+    ~ProfScope();
+    int which;
+    hipStream_t stream;
+    void *slot;
+};
+
 // ---- kernel launchers (one per .hip file) ----------------------------------
 int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
                       int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
@@ -88,8 +98,24 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
     u += 0x7FFFu + ((u >> 16) & 1u);
     return u >> 16;
 }
+// two fp32 -> one dword of two bf16 / two fp16, round to nearest even
+// (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32)
 __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
-    return f32_to_bf16_rne(lo) | (f32_to_bf16_rne(hi) << 16);
+    typedef __attribute__((ext_vector_type(2))) float v2f;
+    typedef __attribute__((ext_vector_type(2))) __bf16 v2b;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f){lo, hi}, v2b));
+}
+__device__ __forceinline__ uint32_t pack_f16_rne(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) float v2f;
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2h;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f){lo, hi}, v2h));
+}
+// Two E4M3 bytes -> one dword of two fp16 (exact: E4M3 fits fp16's normal range)
+template <bool HI>
+__device__ __forceinline__ uint32_t e4m3x2_to_f16x2(uint32_t w) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2h;
+    v2h r = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w, 1.0f, HI);
+    return __builtin_bit_cast(uint32_t, r);
 }
 // Two E4M3 bytes (low or high 16 bits of w) -> two fp32, hardware conversion
 // (OCP E4M3fn on gfx950).

@@ -226,10 +226,16 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     char *ws = (char *)workspace(s, acc_bytes + ml_bytes);
     CWICK_REQUIRE(ws, "gqa_decode: workspace allocation failed");
     float *part_acc = (float *)ws, *part_ml = (float *)(ws + acc_bytes);
-    gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_kv_heads), GQA_DEC_THREADS, 0, s>>>(
-        k, v, q, n_keys, n_kv_heads, (int)per, scale, part_acc, part_ml);
+    {
+        ProfScope ps(CWICK_HIP_PROF_GQA_DECODE, s);
+        gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_kv_heads), GQA_DEC_THREADS, 0, s>>>(
+            k, v, q, n_keys, n_kv_heads, (int)per, scale, part_acc, part_ml);
+    }
     CWICK_HIP_CALL(hipGetLastError());
-    gqa_decode_merge_kernel<HD><<<n_heads, HD, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
+    {
+        ProfScope ps(CWICK_HIP_PROF_GQA_DECODE_MERGE, s);
+        gqa_decode_merge_kernel<HD><<<n_heads, HD, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

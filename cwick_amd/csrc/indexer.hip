@@ -107,8 +107,11 @@ int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_
     indexer_widen_q_kernel<<<(nq + 255) / 256, 256, 0, s>>>(q_idx, nq, qf);
     CWICK_HIP_CALL(hipGetLastError());
     dim3 grid((unsigned)((n_keys + IDX_THREADS - 1) / IDX_THREADS), batch);
-    indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
-                                                       n_keys, qf, w, n_idx_heads, scores);
+    {
+        ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
+        indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
+                                                           n_keys, qf, w, n_idx_heads, scores);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -7,9 +7,10 @@
 //     c_acc[h]     = sum_i p[h][i] * c[sel[i]][0..512)        V = first 512 dims
 //
 // c[t][d] = e4m3(rows[t][d]) * scales[t][d/128].  Every E4M3 value is exact in
-// bf16, so the bytes are widened to bf16 without the scale and the fp32 block
-// scale is applied to the fp32 partial dot of its 128-dim block (scores) or
-// folded into the softmax weight before it is rounded to bf16 (values).
+// bf16 and in fp16, so the bytes are widened without the scale.  Scores: bf16
+// MFMA (the query is bf16), the fp32 block scale multiplies the fp32 partial
+// dot of its 128-dim block.  Values: fp16 MFMA, the block scale is folded into
+// the softmax weight before that is rounded to fp16 (11-bit significand).
 //
 // Work decomposition
 //   workgroup = 256 threads = 4 waves, 32 query rows (heads of one query) x
@@ -42,6 +43,8 @@ constexpr int ROWS = 32;                      // query rows (heads) per workgrou
 constexpr int VT_STRIDE = TK + 8;             // bf16 elements per V^T row (16 B pad)
 constexpr int PS_STRIDE = TK + 8;
 
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
 struct MlaParams {
     const uint8_t *rows;      // [.][n_rows][576]
     const float *scales;      // [.][n_rows][5]
@@ -69,6 +72,7 @@ struct MlaSmem {
     int32_t rowid[TK];                     // cache row of each tile key, -1 = masked
     float wmax[4][ROWS];                   // per-wave tile maxima
     float wsum[4][ROWS];                   // per-wave row sums (epilogue)
+    uint32_t scmax_bits;                   // largest value scale of the tile, as bits
 };
 
 __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams p) {
@@ -127,6 +131,14 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
         for (int h2 = 0; h2 < 2; h2++) oacc[db][h2] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run[2] = {-INFINITY, -INFINITY};
     float l_part[2] = {0.f, 0.f};
+    // The value weights p*scale go through the matrix core as fp16 (11-bit
+    // significand; bf16's 8 bits would cost 2^-9 of the output whenever one key
+    // dominates).  They are kept inside fp16's normal range by a power-of-two
+    // normaliser: e_run is the largest binary exponent of any value scale seen so
+    // far (scale * 2^-e_run < 1), weights are multiplied by 2^(14 - e_run), the
+    // accumulator is in those units and is shifted (exactly) when e_run grows.
+    constexpr int E_NONE = -1000;
+    int e_run = E_NONE;
 
     for (int64_t t0 = k_begin; t0 < k_end; t0 += TK) {
         // ---- tile bookkeeping: cache row and scales of each key ----
@@ -138,12 +150,16 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
                 if (r < 0 || r >= p.n_rows) r = -1;
             }
             sm.rowid[tid] = (int32_t)r;
+            if (tid == 0) sm.scmax_bits = 0u;
         }
         __syncthreads();   // also: everyone is done with the previous tile's LDS
         for (int idx = tid; idx < TK * NBLK; idx += MLA_THREADS) {
             const int key = idx / NBLK, blk = idx % NBLK;
             const int r = sm.rowid[key];
-            sm.sc[key][blk] = r >= 0 ? scales[(size_t)r * NBLK + blk] : 0.0f;
+            const float sv = r >= 0 ? scales[(size_t)r * NBLK + blk] : 0.0f;
+            sm.sc[key][blk] = sv;
+            // positive floats order like their bit patterns
+            if (blk < 4 && sv > 0.0f) atomicMax(&sm.scmax_bits, __builtin_bit_cast(uint32_t, sv));
         }
 
         // ---- this wave's K fragments: issue the loads first ----
@@ -171,11 +187,11 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
 #pragma unroll
                 for (int dw = 0; dw < 4; dw++) {
                     // dims 4dw..4dw+3 of the chunk, for the 4 keys
-                    uint32_t lo[4], hi[4];   // bf16 pairs (dim 4dw,4dw+1) and (4dw+2,4dw+3)
+                    uint32_t lo[4], hi[4];   // fp16 pairs (dim 4dw,4dw+1) and (4dw+2,4dw+3)
 #pragma unroll
                     for (int a = 0; a < 4; a++) {
-                        lo[a] = e4m3x2_to_bf16x2<false>(raw[a][dw]);
-                        hi[a] = e4m3x2_to_bf16x2<true>(raw[a][dw]);
+                        lo[a] = e4m3x2_to_f16x2<false>(raw[a][dw]);
+                        hi[a] = e4m3x2_to_f16x2<true>(raw[a][dw]);
                     }
                     // gather one dim over the 4 keys: low halves, then high halves
                     const int d = chunk * 16 + dw * 4;
@@ -196,6 +212,23 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
             }
         }
         __syncthreads();   // sc[] and vt[] are complete
+
+        // ---- normaliser of the fp16 value weights ----
+        float o_shift = 1.0f;            // exact power of two applied to the accumulator
+        {
+            const uint32_t mb = sm.scmax_bits;
+            const int e_tile = mb ? (int)((mb >> 23) & 0xFFu) - 126 : E_NONE;
+            if (e_tile > e_run) {
+                if (e_run != E_NONE) {
+                    const int d = e_run - e_tile;
+                    o_shift = __builtin_ldexpf(1.0f, d < -120 ? -120 : d);
+                }
+                e_run = e_tile;
+            }
+        }
+        int wexp = 14 - e_run;
+        wexp = wexp > 120 ? 120 : (wexp < -120 ? -120 : wexp);
+        const float wfac = e_run == E_NONE ? 0.0f : __builtin_ldexpf(1.0f, wexp);
 
         // ---- scores for this wave's 16 keys ----
         float s[2][4];
@@ -276,36 +309,46 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
             for (int blk = 0; blk < 4; blk++) {
                 float w[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) w[i] = pv[i] * sm.sc[wave * 16 + 4 * g + i][blk];
+                for (int i = 0; i < 4; i++)
+                    w[i] = pv[i] * (sm.sc[wave * 16 + 4 * g + i][blk] * wfac);   // <= 2^14
                 u32x2 pk;
-                pk[0] = pack_bf16_rne(w[0], w[1]);
-                pk[1] = pack_bf16_rne(w[2], w[3]);
+                pk[0] = pack_f16_rne(w[0], w[1]);
+                pk[1] = pack_f16_rne(w[2], w[3]);
                 *(u32x2 *)&sm.ps[blk][h2 * 16 + l16][wave * 16 + 4 * g] = pk;
             }
         }
 #pragma unroll
-        for (int db = 0; db < 8; db++)
+        for (int h2 = 0; h2 < 2; h2++) {
+            const float oc = corr[h2] * o_shift;
 #pragma unroll
-            for (int h2 = 0; h2 < 2; h2++) oacc[db][h2] *= corr[h2];
+            for (int db = 0; db < 8; db++) oacc[db][h2] *= oc;
+        }
         __syncthreads();   // ps[] complete
 
         // ---- values: dims 128*wave .. 128*wave+127, all TK keys ----
 #pragma unroll
         for (int ks = 0; ks < TK / 32; ks++) {
-            bf16x8 pb[2];
+            f16x8 pb[2];
 #pragma unroll
             for (int h2 = 0; h2 < 2; h2++)
                 pb[h2] = __builtin_bit_cast(
-                    bf16x8, *(const u32x4 *)&sm.ps[wave][h2 * 16 + l16][32 * ks + 8 * g]);
+                    f16x8, *(const u32x4 *)&sm.ps[wave][h2 * 16 + l16][32 * ks + 8 * g]);
 #pragma unroll
             for (int db = 0; db < 8; db++) {
-                const bf16x8 va = __builtin_bit_cast(
-                    bf16x8, *(const u32x4 *)&sm.vt[128 * wave + 16 * db + l16][32 * ks + 8 * g]);
+                const f16x8 va = __builtin_bit_cast(
+                    f16x8, *(const u32x4 *)&sm.vt[128 * wave + 16 * db + l16][32 * ks + 8 * g]);
 #pragma unroll
                 for (int h2 = 0; h2 < 2; h2++)
-                    oacc[db][h2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[h2], oacc[db][h2], 0, 0, 0);
+                    oacc[db][h2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[h2], oacc[db][h2], 0, 0, 0);
             }
         }
+    }
+    // accumulator units -> true units
+    float o_unit = 0.0f;
+    if (e_run != E_NONE) {
+        int ue = e_run - 14;
+        ue = ue > 120 ? 120 : (ue < -120 ? -120 : ue);
+        o_unit = __builtin_ldexpf(1.0f, ue);
     }
 
     // ---- epilogue: row sums over lane groups and waves ----
@@ -325,7 +368,7 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
         const float l = sm.wsum[0][h2 * 16 + l16] + sm.wsum[1][h2 * 16 + l16] +
                         sm.wsum[2][h2 * 16 + l16] + sm.wsum[3][h2 * 16 + l16];
         if (p.n_splits == 1) {
-            const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+            const float inv = l > 0.0f ? o_unit / l : 0.0f;
             float *o = p.out + ((size_t)y * p.nh + head) * VDIM + 128 * wave + 4 * g;
 #pragma unroll
             for (int db = 0; db < 8; db++) *(f32x4 *)(o + 16 * db) = oacc[db][h2] * inv;
@@ -333,7 +376,7 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
             const size_t pr = ((size_t)y * p.n_splits + split) * p.nh + head;
             float *o = p.part_acc + pr * VDIM + 128 * wave + 4 * g;
 #pragma unroll
-            for (int db = 0; db < 8; db++) *(f32x4 *)(o + 16 * db) = oacc[db][h2];
+            for (int db = 0; db < 8; db++) *(f32x4 *)(o + 16 * db) = oacc[db][h2] * o_unit;
             if (wave == 0 && g == 0) {
                 p.part_ml[pr * 2 + 0] = m_run[h2];
                 p.part_ml[pr * 2 + 1] = l;
@@ -386,9 +429,13 @@ static int run_mla(MlaParams &p, hipStream_t s) {
         p.part_acc = (float *)ws;
         p.part_ml = (float *)(ws + acc_b);
     }
-    mla_fwd_kernel<<<dim3((unsigned)total), MLA_THREADS, smem, s>>>(p);
+    {
+        ProfScope ps(CWICK_HIP_PROF_MLA, s);
+        mla_fwd_kernel<<<dim3((unsigned)total), MLA_THREADS, smem, s>>>(p);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
+        ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
         mla_merge_kernel<<<dim3(p.nh, p.nq), 256, 0, s>>>(p.part_acc, p.part_ml, p.n_splits, p.nh, p.out);
         CWICK_HIP_CALL(hipGetLastError());
     }

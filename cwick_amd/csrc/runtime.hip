@@ -11,6 +11,7 @@
 #include <string>
 #include <strings.h>
 #include <unordered_map>
+#include <vector>
 
 namespace cwick {
 
@@ -125,6 +126,61 @@ static void *grow(std::unordered_map<hipStream_t, Scratch> &m, hipStream_t s, si
 
 void *workspace(hipStream_t s, size_t bytes) { return grow(g_ws, s, bytes); }
 void *staging(hipStream_t s, size_t bytes) { return grow(g_stage, s, bytes); }
+
+// ---------------------------------------------------------------------------
+// phase timers: event pairs around kernel launches, summed on read
+// ---------------------------------------------------------------------------
+struct ProfPair {
+    hipEvent_t a, b;
+    int which;
+};
+static std::mutex g_prof_mu;
+static bool g_prof_on = false;
+static std::vector<ProfPair> g_prof_pending;       // recorded, not yet summed
+static std::vector<ProfPair> g_prof_free;          // reusable event pairs
+static double g_prof_ms[CWICK_HIP_PROF_COUNT];
+static int64_t g_prof_n[CWICK_HIP_PROF_COUNT];
+
+ProfScope::ProfScope(int w, hipStream_t s) : which(w), stream(s), slot(nullptr) {
+    if (!g_prof_on) return;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfPair *pp = new ProfPair;
+    if (!g_prof_free.empty()) {
+        *pp = g_prof_free.back();
+        g_prof_free.pop_back();
+    } else if (hipEventCreate(&pp->a) != hipSuccess || hipEventCreate(&pp->b) != hipSuccess) {
+        (void)hipGetLastError();
+        delete pp;
+        return;
+    }
+    pp->which = w;
+    (void)hipEventRecord(pp->a, s);
+    slot = pp;
+}
+
+ProfScope::~ProfScope() {
+    if (!slot) return;
+    ProfPair *pp = (ProfPair *)slot;
+    (void)hipEventRecord(pp->b, stream);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_pending.push_back(*pp);
+    delete pp;
+}
+
+static void prof_drain_locked() {
+    for (ProfPair &pp : g_prof_pending) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(pp.b) == hipSuccess &&
+            hipEventElapsedTime(&ms, pp.a, pp.b) == hipSuccess) {
+            g_prof_ms[pp.which] += (double)ms;
+            g_prof_n[pp.which] += 1;
+        } else {
+            (void)hipGetLastError();
+        }
+        g_prof_free.push_back(pp);
+    }
+    g_prof_pending.clear();
+}
 
 static void free_all_scratch() {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -703,6 +759,37 @@ int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, 
     CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
     if (sel_out) CWICK_HIP_CALL(hipMemcpy(sel_out, dsel, selb, hipMemcpyDeviceToHost));
     return 1;
+}
+
+void cwick_hip_prof_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_on = on != 0;
+}
+
+void cwick_hip_prof_reset(void) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    prof_drain_locked();
+    for (int i = 0; i < CWICK_HIP_PROF_COUNT; i++) {
+        g_prof_ms[i] = 0.0;
+        g_prof_n[i] = 0;
+    }
+}
+
+int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches) {
+    clear_error();
+    CWICK_REQUIRE(which >= 0 && which < CWICK_HIP_PROF_COUNT, "prof_read: unknown timer %d", which);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    prof_drain_locked();
+    if (total_ms) *total_ms = g_prof_ms[which];
+    if (launches) *launches = g_prof_n[which];
+    return 1;
+}
+
+const char *cwick_hip_prof_name(int which) {
+    static const char *names[CWICK_HIP_PROF_COUNT] = {
+        "gqa_decode_split_kernel", "gqa_decode_merge_kernel", "gqa_prefill_kernel",
+        "mla_fwd_kernel", "mla_merge_kernel", "indexer_scores_kernel", "topk_radix_kernel"};
+    return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 
 int cwick_hip_e4m3_table(float *out256) {

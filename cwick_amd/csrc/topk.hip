@@ -165,7 +165,10 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     CWICK_REQUIRE(batch >= 1 && batch <= 65535, "topk: batch %d", batch);
     CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
-    topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+    {
+        ProfScope ps(CWICK_HIP_PROF_TOPK, s);
+        topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -74,6 +74,10 @@ SIGNATURES = {
                                         _vp, _vp, _int, _i64, _vp, _int, _flt, _vp, _vp, _vp,
                                         _vp]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
+    "cwick_hip_prof_enable": (None, [_int]),
+    "cwick_hip_prof_reset": (None, []),
+    "cwick_hip_prof_read": (_int, [_int, C.POINTER(C.c_double), C.POINTER(_i64)]),
+    "cwick_hip_prof_name": (C.c_char_p, [_int]),
 }
 
 
@@ -396,3 +400,27 @@ def dsa_decode_dev(ikeys, ikscale, key_bstride, kscale_bstride, rows, scales, ro
         row_bstride, scale_bstride, batch, n_keys, _dp(q_idx), _dp(w), n_idx_heads, topk_k,
         _dp(q), n_heads, scale, _dp(scores_tmp), _dp(sel_out), _dp(out), stream),
         "dsa_decode_dev")
+
+
+# ------------------------------------------------------------------ phase timers
+PROF_NAMES = ["gqa_decode_split_kernel", "gqa_decode_merge_kernel", "gqa_prefill_kernel",
+              "mla_fwd_kernel", "mla_merge_kernel", "indexer_scores_kernel", "topk_radix_kernel"]
+
+
+def prof_enable(on=True):
+    lib().cwick_hip_prof_enable(1 if on else 0)
+
+
+def prof_reset():
+    lib().cwick_hip_prof_reset()
+
+
+def prof_read():
+    """{kernel name: (total_ms, launches)} since the last reset (waits for the GPU)."""
+    out = {}
+    for i, name in enumerate(PROF_NAMES):
+        ms, n = C.c_double(0.0), _i64(0)
+        _check(lib().cwick_hip_prof_read(i, C.byref(ms), C.byref(n)), "prof_read")
+        assert lib().cwick_hip_prof_name(i).decode() == name
+        out[name] = (ms.value, n.value)
+    return out

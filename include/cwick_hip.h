@@ -241,6 +241,29 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale,
                              float scale, float *scores_tmp, int32_t *sel_out, float *out,
                              void *stream);
 
+/* ---- phase timers ------------------------------------------------------- */
+/* Replace the reference's attention sub-timers (g_attn_*_ns, src/attention.c:1169-1174,
+ * read out by src/prof.c:184-196 under CWICK_PROFILE; CWICK_Q35_PROF's
+ * qk/softmax/av split, src/q35_model.c:72-99).  While enabled, every launch of
+ * a kernel listed below is bracketed by a pair of HIP events on the stream it
+ * is launched on; cwick_hip_prof_read() waits for the recorded events and
+ * returns the summed GPU time and the number of launches since the last reset.
+ * Off by default (no events are recorded). */
+enum {
+    CWICK_HIP_PROF_GQA_DECODE = 0,      /* gqa_decode_split_kernel */
+    CWICK_HIP_PROF_GQA_DECODE_MERGE,    /* gqa_decode_merge_kernel */
+    CWICK_HIP_PROF_GQA_PREFILL,         /* gqa_prefill_kernel */
+    CWICK_HIP_PROF_MLA,                 /* mla_fwd_kernel (decode, sparse, prefill) */
+    CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_kernel */
+    CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel */
+    CWICK_HIP_PROF_TOPK,                /* topk_radix_kernel */
+    CWICK_HIP_PROF_COUNT
+};
+void cwick_hip_prof_enable(int on);
+void cwick_hip_prof_reset(void);
+int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches);
+const char *cwick_hip_prof_name(int which);
+
 /* Device-side codec check used by the parity tests: decodes all 256 E4M3
  * bytes with the conversion instruction the kernels use into out256 (host). */
 int cwick_hip_e4m3_table(float *out256);

@@ -33,19 +33,31 @@ def hip():
 # Tolerance of the attention outputs against the CPU oracle: max-abs 2e-3 and
 # max-abs / max|reference| 1e-2 (the form the reference's own self-check prints,
 # src/attention.c:881-891).
+#
+# strict=True (the five benchmark configurations and everything shaped like them):
+#     max|got-ref| <= 2e-3  AND  max|got-ref| / max|ref| <= 1e-2.
+# strict=False (edge cases whose outputs are O(1), e.g. a single key, where the
+# output IS a latent value and a bf16-rounded weight alone moves it by 2^-9 of
+# itself): the elementwise form |got-ref| <= 2e-3 + 1e-2*|ref|.
 ATOL, RTOL = 2e-3, 1e-2
 
 
-def assert_close(got, ref, what=""):
+def assert_close(got, ref, what="", strict=True):
     import numpy as np
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     assert got.shape == ref.shape, (got.shape, ref.shape)
     assert np.isfinite(got).all(), what + ": non-finite output"
-    diff = np.abs(got - ref).max()
+    err = np.abs(got - ref)
+    diff = err.max()
     refmax = np.abs(ref).max()
     rel = diff / refmax if refmax > 0 else diff
-    print("[parity] %-40s maxabs %.3e  rel %.3e  refmax %.3e" % (what, diff, rel, refmax),
-          flush=True)
-    assert diff <= ATOL, "%s: max-abs %.3e > %.1e" % (what, diff, ATOL)
-    assert rel <= RTOL, "%s: rel %.3e > %.1e" % (what, rel, RTOL)
+    print("[parity] %-44s maxabs %.3e  rel %.3e  refmax %.3e%s" %
+          (what, diff, rel, refmax, "" if strict else "  (elementwise)"), flush=True)
+    if strict:
+        assert diff <= ATOL, "%s: max-abs %.3e > %.1e" % (what, diff, ATOL)
+        assert rel <= RTOL, "%s: rel %.3e > %.1e" % (what, rel, RTOL)
+    else:
+        bad = err > ATOL + RTOL * np.abs(ref)
+        assert not bad.any(), "%s: %d elements outside 2e-3 + 1e-2*|ref| (max-abs %.3e)" % (
+            what, int(bad.sum()), diff)
