@@ -37,8 +37,8 @@ def _hipcc():
 def _compile(src, force):
     obj = os.path.join(OBJDIR, src.replace(".hip", ".o"))
     path = os.path.join(CSRC, src)
-    deps = [path, os.path.join(CSRC, "common.hpp"),
-            os.path.join(HERE, "..", "include", "cwick_hip.h"), os.path.abspath(__file__)]
+    deps = [path, os.path.join(HERE, "..", "include", "cwick_hip.h"), os.path.abspath(__file__)]
+    deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
     if not force and os.path.exists(obj) and all(
             os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj, ""

@@ -18,6 +18,7 @@
 //   the rescale; the lane groups of a workgroup are merged through LDS, then
 //   (m, l, acc) goes to the workspace and a second kernel merges the splits.
 #include "common.hpp"
+#include "merge.hpp"
 
 namespace cwick {
 
@@ -189,25 +190,6 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
     }
 }
 
-// out[h][d] = sum_s acc_s[h][d] e^{m_s - M} / sum_s l_s e^{m_s - M}
-template <int HD>
-__global__ void __launch_bounds__(HD)
-gqa_decode_merge_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
-                        int n_splits, int n_heads, float *__restrict__ out) {
-    const int h = blockIdx.x, d = threadIdx.x;
-    float mx = -INFINITY;
-    for (int s = 0; s < n_splits; s++) mx = fmaxf(mx, part_ml[((size_t)s * n_heads + h) * 2]);
-    float a = 0.0f, l = 0.0f;
-    for (int s = 0; s < n_splits; s++) {
-        const float ms = part_ml[((size_t)s * n_heads + h) * 2];
-        if (ms == -INFINITY) continue;
-        const float c = __expf(ms - mx);
-        a += part_acc[((size_t)s * n_heads + h) * HD + d] * c;
-        l += part_ml[((size_t)s * n_heads + h) * 2 + 1] * c;
-    }
-    out[(size_t)h * HD + d] = a / l;
-}
-
 template <int HD, int GROUP>
 static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
                           const uint16_t *q, float scale, float *out, hipStream_t s) {
@@ -217,6 +199,7 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     // enough workgroups for ~2 per CU, each at least one full step
     int64_t want = (int64_t)2 * num_cus() / n_kv_heads;
     if (want < 1) want = 1;
+    if (want > MERGE_MAX_SPLITS) want = MERGE_MAX_SPLITS;
     int64_t per = (n_keys + want - 1) / want;
     per = ((per + step - 1) / step) * step;
     if (per < step) per = step;
@@ -234,7 +217,7 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     CWICK_HIP_CALL(hipGetLastError());
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_DECODE_MERGE, s);
-        gqa_decode_merge_kernel<HD><<<n_heads, HD, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
+        splitk_merge_kernel<HD><<<dim3(n_heads, 1), 256, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

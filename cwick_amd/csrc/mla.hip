@@ -31,6 +31,7 @@
 //            combines them.  prefill: one workgroup walks the whole causal
 //            prefix of its query and writes the normalised output.
 #include "common.hpp"
+#include "merge.hpp"
 
 namespace cwick {
 
@@ -385,31 +386,6 @@ __global__ void __launch_bounds__(MLA_THREADS, 1) mla_fwd_kernel(const MlaParams
     }
 }
 
-// out[y][h][d] = sum_s acc_s e^{m_s - M} / sum_s l_s e^{m_s - M}
-__global__ void __launch_bounds__(256)
-mla_merge_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
-                 int n_splits, int nh, float *__restrict__ out) {
-    const int h = blockIdx.x, y = blockIdx.y;
-    const size_t base = (size_t)y * n_splits;
-    float mx = -INFINITY;
-    for (int s = 0; s < n_splits; s++) mx = fmaxf(mx, part_ml[((base + s) * nh + h) * 2]);
-    float a0 = 0.f, a1 = 0.f, l = 0.f;
-    const int d = threadIdx.x;
-    for (int s = 0; s < n_splits; s++) {
-        const size_t pr = (base + s) * nh + h;
-        const float ms = part_ml[pr * 2];
-        if (ms == -INFINITY) continue;
-        const float c = __expf(ms - mx);
-        a0 += part_acc[pr * VDIM + d] * c;
-        a1 += part_acc[pr * VDIM + 256 + d] * c;
-        l += part_ml[pr * 2 + 1] * c;
-    }
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    float *o = out + ((size_t)y * nh + h) * VDIM;
-    o[d] = a0 * inv;
-    o[256 + d] = a1 * inv;
-}
-
 static int run_mla(MlaParams &p, hipStream_t s) {
     static bool attr_set = false;
     const size_t smem = sizeof(MlaSmem);
@@ -436,7 +412,7 @@ static int run_mla(MlaParams &p, hipStream_t s) {
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
         ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
-        mla_merge_kernel<<<dim3(p.nh, p.nq), 256, 0, s>>>(p.part_acc, p.part_ml, p.n_splits, p.nh, p.out);
+        splitk_merge_kernel<VDIM><<<dim3(p.nh, p.nq), 256, 0, s>>>(p.part_acc, p.part_ml, p.n_splits, p.nh, p.out);
         CWICK_HIP_CALL(hipGetLastError());
     }
     return 1;
