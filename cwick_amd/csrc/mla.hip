@@ -418,7 +418,7 @@ static int run_mla(MlaParams &p, hipStream_t s) {
     return 1;
 }
 
-int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
+int launch_mla_decode_v1(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
                       int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
                       hipStream_t s) {
@@ -450,7 +450,7 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
     return run_mla(p, s);
 }
 
-int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+int launch_mla_prefill_v1(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
                        const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s) {
     CWICK_REQUIRE(rows && scales && q && out, "mla_prefill: null pointer");
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill: n_heads %d (1..128)", n_heads);
