@@ -3,23 +3,38 @@
 // per 128-query tile S = scale*Q*K^T over the rectangle, -1e30 tail, softmax,
 // O = S*V).  Here: one pass, online softmax, the triangle only.
 //
-// MFMA-bound.  Work decomposition
-//   workgroup = 4 waves = 128 query rows that share one kv head: the GROUP
-//   query heads of the kv head times P = 128/GROUP consecutive positions
+// MFMA-bound, and on this machine that means LDS-aware: a 32x32x16 MFMA takes
+// 32 cycles and its A operand is 1 KiB, so four SIMDs that each fetch their own
+// A fragments need the whole 128 B/clk of LDS.  Every wave therefore owns 64
+// query rows (two 32-row column blocks) and uses each K / V^T fragment twice.
+//
+//   workgroup = 4 waves = 256 query rows that share one kv head: the GROUP
+//   query heads of the kv head times P = 256/GROUP consecutive positions
 //   (heads-as-M: K and V tiles are read once for all heads of the group).
-//   wave = 32 rows.  Key tiles of TK = 32, K and V copied global -> LDS as they
-//   are ([key][dim] bf16, double buffered, next tile prefetched in registers).
+//   Key tiles of TK = 32.  K and V go global -> LDS by global_load_lds_dwordx4
+//   (no staging registers), two tiles ahead for K and one for V, one workgroup
+//   barrier per tile.
 //   scores:  S^T[key][row] = K[key][dim] . Q^T[dim][row], v_mfma_f32_32x32x16_bf16,
-//            K fragments from LDS, Q fragments resident in registers.
+//            K fragments from LDS, Q fragments resident in registers (80 of 128; the rest re-read from LDS).
 //            One query row per lane column: softmax statistics are per-lane.
 //   values:  O^T[dim][row] += V^T[dim][key] . P^T[key][row].  P^T is the score
 //            accumulator itself (rounded to bf16) -- its register layout is the
 //            B-operand layout once the contraction slots are numbered to match;
-//            V^T fragments come out of the row-major V tile through the LDS
-//            transpose read (ds_read_b64_tr_b16), so nothing is transposed by hand.
-//   The running maximum is only advanced when a tile beats it by more than 8
-//   (in log2 units), so the 128 output registers are rescaled a few times per
-//   row block instead of once per tile.
+//            V^T fragments come out of the V tile through the LDS transpose read
+//            (ds_read_b64_tr_b16).  The 256 output registers live in AGPRs.
+//   schedule: one wave per SIMD, so the loop is software-pipelined by hand: the
+//            body computes the scores of tile t+1, and then the softmax of tile
+//            t+1 (VALU) next to the value MFMAs of tile t.
+//   The softmax reference of a row is the maximum of its first tile and stays
+//   there while later scores exceed it by less than 64 (log2 units): weights up
+//   to 2^64 lose nothing in bf16 or fp32.  A wave that meets a larger score
+//   leaves the fast loop for a slow one that moves the reference and rescales
+//   the accumulators (in place, in AGPRs) every tile.
+//
+//   LDS tile layout: 16 blocks of 1 KiB (+64 B pad), block b = 16-byte columns
+//   2b and 2b+1 of all 32 keys, slot (c&1)*32 + (key ^ 8(c&1)).  A K fragment
+//   read (ds_read_b128) covers one whole block; a transpose read touches four
+//   64-byte segments that fall into different banks.
 #include "common.hpp"
 
 namespace cwick {
@@ -27,68 +42,74 @@ namespace cwick {
 constexpr int PF_THREADS = 256;
 constexpr int PF_TK = 32;
 constexpr int PF_HD = 256;
-constexpr int PF_LD = PF_HD + 8;            // LDS row stride in bf16 (16 B pad)
-constexpr int PF_ROWS = 128;                // query rows per workgroup
-// Resident workgroups per CU the register budget is sized for: 1 leaves each
-// wave the whole 512-register file (Q fragments 64 + output 128 + staging),
-// 2 would need the kernel to fit 256 and spills today.
-constexpr int PF_WG_PER_CU = 1;
+constexpr int PF_ROWS = 256;                // query rows per workgroup
+constexpr int PF_BLK = 1024 + 64;           // bytes between LDS blocks
+constexpr int PF_TILE = 16 * PF_BLK;        // one K or V tile in LDS
+constexpr int PF_PRE = 4;                   // k-steps of fragment prefetch in the score loop
+constexpr int PF_QX0 = 0;                   // first k-step of column block B whose Q fragment is parked in LDS
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef __attribute__((address_space(3))) void pf_lds_void;
 
 struct PfSmem {
-    uint16_t k[2][PF_TK][PF_LD];
-    uint16_t v[2][PF_TK][PF_LD];
+    unsigned char k[2][PF_TILE];
+    unsigned char v[2][PF_TILE];
+    // Q fragments of column block B, k-steps PF_QX0..15, parked per lane: the register file
+    // holds 256 accumulators + 80 Q registers + the working set, not 128 Q registers
+    u32x4 qx[PF_THREADS / 64][16 - PF_QX0][64];
 };
 
-template <int GROUP>
-__global__ void __launch_bounds__(PF_THREADS, PF_WG_PER_CU)
+// workgroup barrier that orders LDS traffic only (the copies of later tiles stay in flight)
+#define PF_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+// PRECISE: the bf16 rounding residual of the weights goes through the matrix core as well
+// (position blocks that see at most 2048 keys; see the launcher).
+template <int GROUP, bool PRECISE>
+__global__ void __launch_bounds__(PF_THREADS, 1)
 gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
                    const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
-                   float scale_log2e, float *__restrict__ out) {
+                   float scale_log2e, float *__restrict__ out, int64_t pblk_lo) {
     constexpr int P = PF_ROWS / GROUP;      // positions per workgroup
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     PfSmem &sm = *reinterpret_cast<PfSmem *>(smem_raw);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31;
     const int g = lane >> 5;                // 0/1
 
     const int kvh = blockIdx.y;
     // heavy (late) position blocks first: better tail balance under the causal triangle
-    const int64_t pblk = (int64_t)gridDim.x - 1 - blockIdx.x;
+    const int64_t pblk = pblk_lo + ((int64_t)gridDim.x - 1 - blockIdx.x);
     const int64_t t0 = pblk * P;
     const int n_heads = n_kv_heads * GROUP;
     const int64_t kv_stride = (int64_t)n_kv_heads * PF_HD;
     const int64_t q_stride = (int64_t)n_heads * PF_HD;
     const int64_t n_keys_all = pos0 + n;
 
-    // this lane's query row
-    const int r = wave * 32 + l32;
-    const int j = r / P;                    // head within the group
-    const int64_t t = t0 + (r % P);         // position within the chunk
-    const bool row_live = t < n;
-    const int64_t tq = row_live ? t : n - 1;
-    const int64_t my_limit = pos0 + tq;     // last visible key
-
-    // Q fragments: B operand, lane (row, g) holds dims 16ks+8g .. +8
-    bf16x8 qf[16];
-    {
-        const uint16_t *qrow = Q + tq * q_stride + (size_t)(kvh * GROUP + j) * PF_HD + 8 * g;
+    // this lane's two query rows (column blocks A and B of the wave)
+    int64_t t_row[2], my_limit[2];
+    int j_row[2];
+    bool row_live[2];
+    bf16x8 qf[2][16];                       // B operand: lane (row, g) holds dims 16ks+8g .. +8
+                                            // (qf[1][PF_QX0..15] only pass through, see PfSmem::qx)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int r = wave * 64 + 32 * c + l32;
+        j_row[c] = r / P;
+        t_row[c] = t0 + (r % P);
+        row_live[c] = t_row[c] < n;
+        const int64_t tq = row_live[c] ? t_row[c] : n - 1;
+        my_limit[c] = pos0 + tq;
+        const uint16_t *qrow = Q + tq * q_stride + (size_t)(kvh * GROUP + j_row[c]) * PF_HD + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < 16; ks++)
-            qf[ks] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qrow + 16 * ks));
+            qf[c][ks] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qrow + 16 * ks));
     }
-
-    f32x16 oacc[8];
 #pragma unroll
-    for (int db = 0; db < 8; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] = 0.0f;
-    float m_ref = -INFINITY, l_part = 0.0f;
+    for (int ks = PF_QX0; ks < 16; ks++) sm.qx[wave][ks - PF_QX0][lane] = __builtin_bit_cast(u32x4, qf[1][ks]);
 
     // keys 0 .. last position of the block (clipped to the chunk)
     int64_t last_t = t0 + P - 1;
@@ -96,152 +117,273 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     const int64_t wg_keys = pos0 + last_t + 1;
     const int n_tiles = (int)((wg_keys + PF_TK - 1) / PF_TK);
     const int64_t first_masked_key = pos0 + t0;   // tiles ending at or below this need no mask
-    const bool precise = wg_keys <= 2048;         // workgroup-uniform
+    constexpr bool precise = PRECISE;
 
-    const uint16_t *Kg = K + (size_t)kvh * PF_HD;
-    const uint16_t *Vg = V + (size_t)kvh * PF_HD;
-
-    // global -> register staging of one tile: 32 rows x 512 B, 4 x 16 B per thread
-    // One set of staging registers serves K (in flight during the score MFMAs)
-    // and then V (in flight during softmax and the value MFMAs).
-    u32x4 st[4];
-    auto load_rows = [&](const uint16_t *base, int tile) {
+    // ---- global -> LDS copies.  Wave w copies blocks 4w..4w+3 of a tile; lane l of a copy
+    // lands in slot l of the block: column 2b + (l>>5), key (l&31) ^ 8(l>>5).
+    const int cp_key = l32 ^ (g << 3);
+    const uint16_t *Kg = K + (size_t)kvh * PF_HD + 8 * g;
+    const uint16_t *Vg = V + (size_t)kvh * PF_HD + 8 * g;
+    const uint32_t lds_k = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.k[0][0];
+    const uint32_t lds_v = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.v[0][0];
+    auto issue = [&](const uint16_t *base, uint32_t lds_tile, int tile) {
+        int64_t row = (int64_t)tile * PF_TK + cp_key;
+        if (row > n_keys_all - 1) row = n_keys_all - 1;         // masked anyway
+        const uint16_t *src = base + row * kv_stride + 64 * wave;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int c = tid + PF_THREADS * i;
-            int64_t row = (int64_t)tile * PF_TK + (c >> 5);
-            if (row > n_keys_all - 1) row = n_keys_all - 1;     // masked anyway
-            st[i] = *(const u32x4 *)(base + row * kv_stride + (c & 31) * 8);
-        }
-    };
-    auto store_rows = [&](uint16_t (*dst)[PF_LD]) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + PF_THREADS * i;
-            *(u32x4 *)&dst[c >> 5][(c & 31) * 8] = st[i];
+            const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK));
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         ::"v"(src + 16 * i), "s"(off) : "memory");
         }
     };
 
-    load_rows(Kg, 0);
-    store_rows(sm.k[0]);
-    load_rows(Vg, 0);
-    store_rows(sm.v[0]);
-    __syncthreads();
-
-    for (int tile = 0; tile < n_tiles; tile++) {
-        const int buf = tile & 1;
-        const bool more = tile + 1 < n_tiles;
-        if (more) load_rows(Kg, tile + 1);
-
-        // ---- scores: S^T[32 keys][32 rows] ----
-        f32x16 s;
+    // K fragment of k-step ks: block ks, slot 32g + (l32 ^ 8g)
+    const uint32_t kfrag_off = (uint32_t)((32 * g + (l32 ^ (g << 3))) * 16);
+    // transpose read (ds_read_b64_tr_b16): within a 16-lane group, lane i addresses key (i/4),
+    // dims 4*(i%4)..+4 of a 4-key x 16-dim patch and receives dim i for the 4 keys.
+    // For output block db: dims 32db + 16(grp&1) + 4(gi&3): column c = 4db + 2(grp&1) + ((gi&3)>>1)
+    const int grp = lane >> 4, gi = lane & 15;
+    const int v_col = (gi & 3) >> 1;                              // parity of the 16-byte column
+    const int v_key0 = 4 * (grp >> 1) + (gi >> 2);                // + 16 ks2 (+8 for the second half)
+    auto vfrag_off = [&](int key) -> uint32_t {
+        return (uint32_t)((grp & 1) * PF_BLK + (v_col * 32 + (key ^ (v_col << 3))) * 16 + (gi & 1) * 8);
+    };
+    uint32_t v_off[2][2];
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < 16; ks++) {
-            const bf16x8 ka = __builtin_bit_cast(bf16x8, *(const u32x4 *)&sm.k[buf][l32][16 * ks + 8 * g]);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], s, 0, 0, 0);
-        }
-        if (more) {
-            store_rows(sm.k[buf ^ 1]);
-            load_rows(Vg, tile + 1);
-        }
-        // register i holds key (i/4)*8 + 4g + i%4 of the tile for this lane's row
-        const int64_t key0 = (int64_t)tile * PF_TK;
-        const bool need_mask = key0 + PF_TK - 1 > first_masked_key;
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float x = s[i] * scale_log2e;
-            if (need_mask) {
-                const int64_t key = key0 + (i >> 2) * 8 + 4 * g + (i & 3);
-                if (key > my_limit) x = -INFINITY;
-            }
-            s[i] = x;
-            tmax = fmaxf(tmax, x);
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        if (__any(tmax > m_ref + 8.0f)) {
-            const float m_new = fmaxf(m_ref, tmax);
-            const float corr = __builtin_amdgcn_exp2f(m_ref - m_new);       // first tile: exp2(-inf) = 0
-            m_ref = m_new;
-            l_part *= corr;
-#pragma unroll
-            for (int db = 0; db < 8; db++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) oacc[db][i] *= corr;
-        }
-        float psum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            s[i] = __builtin_amdgcn_exp2f(s[i] - m_ref);                    // masked: 0
-            psum += s[i];
-        }
-        l_part += psum;
-
-        // ---- values: two k-steps of 16 keys ----
-        // contraction slot (g, jj) of step ks2 <-> tile key 16*ks2 + (jj/4)*8 + 4g + jj%4,
-        // i.e. score register 8*ks2 + jj: P^T needs no data movement.
-#pragma unroll
-        for (int ks2 = 0; ks2 < 2; ks2++) {
-            u32x4 pw;
-#pragma unroll
-            for (int h = 0; h < 4; h++)
-                pw[h] = pack_bf16_rne(s[8 * ks2 + 2 * h], s[8 * ks2 + 2 * h + 1]);
-            const bf16x8 pb = __builtin_bit_cast(bf16x8, pw);
-            // Short prefixes: few keys carry the whole weight, so the 2^-9 rounding of
-            // each bf16 weight shows in an O(1) output.  There the rounding residual
-            // goes through the matrix core as well (weights good to 2^-17).
-            bf16x8 pb_lo = pb;
-            if (precise) {
-                u32x4 pl;
-#pragma unroll
-                for (int h = 0; h < 4; h++)
-                    pl[h] = pack_bf16_rne(s[8 * ks2 + 2 * h] - bf16lo_to_f32(pw[h]),
-                                          s[8 * ks2 + 2 * h + 1] - bf16hi_to_f32(pw[h]));
-                pb_lo = __builtin_bit_cast(bf16x8, pl);
-            }
-            // transpose read: within a 16-lane group, lane i addresses key (i/4), dims
-            // 4*(i%4)..+4 of a 4 x 16 tile and receives dim (i) for the 4 keys.
-            const int grp = lane >> 4;                    // 16-lane group 0..3
-            const int gi = lane & 15;
-            const int dim_in = 16 * (grp & 1) + 4 * (gi & 3);
-            const int key_a = 16 * ks2 + 4 * (grp >> 1) + (gi >> 2);   // slots jj = 0..3
-            const int key_b = key_a + 8;                                // slots jj = 4..7
-#pragma unroll
-            for (int db = 0; db < 8; db++) {
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (lds_s16x4 *)&sm.v[buf][key_a][32 * db + dim_in]);
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (lds_s16x4 *)&sm.v[buf][key_b][32 * db + dim_in]);
-                typedef __attribute__((ext_vector_type(8))) short s16x8;
-                const s16x8 va8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va8), pb,
-                                                                   oacc[db], 0, 0, 0);
-                if (precise)
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, va8), pb_lo, oacc[db], 0, 0, 0);
-            }
-        }
-
-        if (more) store_rows(sm.v[buf ^ 1]);
-        __syncthreads();
+    for (int ks2 = 0; ks2 < 2; ks2++) {
+        v_off[ks2][0] = vfrag_off(16 * ks2 + v_key0);
+        v_off[ks2][1] = vfrag_off(16 * ks2 + v_key0 + 8);
     }
 
-    // ---- epilogue ----
-    const float l = l_part + __shfl_xor(l_part, 32, 64);
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (row_live) {
-        float *o = out + t * q_stride + (size_t)(kvh * GROUP + j) * PF_HD + 4 * g;
+    f32x16 oacc[2][8];
+#pragma unroll
+    for (int c = 0; c < 2; c++)
 #pragma unroll
         for (int db = 0; db < 8; db++)
 #pragma unroll
-            for (int b4 = 0; b4 < 4; b4++) {
-                f32x4 w;
+            for (int i = 0; i < 16; i++) oacc[c][db][i] = 0.0f;
+    float m_ref[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.0f, 0.0f};
+
+    // scores of one tile for both column blocks
+    // One wave per SIMD: nothing hides an LDS round trip, so the fragments are fetched PF_PRE
+    // k-steps ahead of the MFMAs that use them.
+    auto scores = [&](int tile, f32x16 (&s)[2]) {
+        const unsigned char *kb = &sm.k[tile & 1][0] + kfrag_off;
+        const u32x4 *qb = &sm.qx[wave][0][lane];
+        u32x4 ka[PF_PRE], qa[PF_PRE];
 #pragma unroll
-                for (int i = 0; i < 4; i++) w[i] = oacc[db][4 * b4 + i] * inv;
-                *(f32x4 *)(o + 32 * db + 8 * b4) = w;
+        for (int ks = 0; ks < PF_PRE; ks++) {
+            ka[ks] = *(const u32x4 *)(kb + ks * PF_BLK);
+            if (ks >= PF_QX0) qa[ks] = qb[(ks - PF_QX0) * 64];
+        }
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[c][i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            const bf16x8 kf = __builtin_bit_cast(bf16x8, ka[ks % PF_PRE]);
+            const bf16x8 q1 = ks < PF_QX0 ? qf[1][ks] : __builtin_bit_cast(bf16x8, qa[ks % PF_PRE]);
+            if (ks + PF_PRE < 16) {
+                ka[ks % PF_PRE] = *(const u32x4 *)(kb + (ks + PF_PRE) * PF_BLK);
+                if (ks + PF_PRE >= PF_QX0) qa[ks % PF_PRE] = qb[(ks + PF_PRE - PF_QX0) * 64];
             }
+            s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
+            s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q1, s[1], 0, 0, 0);
+        }
+    };
+    // softmax bookkeeping of one tile and column block, in two parts.
+    // register i holds key (i/4)*8 + 4g + i%4 of the tile for this lane's row.
+    // sm_prep: mask the raw scores, return this lane's maximum in log2 units.
+    auto sm_prep = [&](int tile, int c, f32x16 &s) -> float {
+        const int64_t key0 = (int64_t)tile * PF_TK;
+        float tmax = -INFINITY;
+        if (key0 + PF_TK - 1 > first_masked_key) {          // workgroup-uniform: a tile on the diagonal
+            // position (i/4)*8 + i%4 + 4g of the tile is visible up to lim
+            int64_t lim64 = my_limit[c] - key0 - 4 * g;
+            const int lim = lim64 > 64 ? 64 : (lim64 < -1 ? -1 : (int)lim64);
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                if ((i >> 2) * 8 + (i & 3) > lim) s[i] = -INFINITY;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[i]);
+        return tmax * scale_log2e;                           // the scale is positive: max commutes
+    };
+    // sm_finish: raw scores -> bf16 weights (and their rounding residual) against m_ref.
+    auto sm_finish = [&](int c, f32x16 &s, u32x4 (&pw)[2], u32x4 (&pl)[2]) {
+        const float m_use = m_ref[c] == -INFINITY ? 0.0f : m_ref[c];
+        float psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            s[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale_log2e, -m_use));   // masked: 0
+            psum += s[i];
+        }
+        l_part[c] += psum;
+        // contraction slot (g, jj) of step ks2 <-> tile key 16*ks2 + (jj/4)*8 + 4g + jj%4,
+        // i.e. score register 8*ks2 + jj: P^T needs no data movement.
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ks2++)
+#pragma unroll
+            for (int h = 0; h < 4; h++) {
+                pw[ks2][h] = pack_bf16_rne(s[8 * ks2 + 2 * h], s[8 * ks2 + 2 * h + 1]);
+                if (precise)
+                    pl[ks2][h] = pack_bf16_rne(s[8 * ks2 + 2 * h] - bf16lo_to_f32(pw[ks2][h]),
+                                               s[8 * ks2 + 2 * h + 1] - bf16hi_to_f32(pw[ks2][h]));
+            }
+    };
+    // The running reference m_ref is the row maximum of tile 0 and stays there while later tiles
+    // exceed it by less than 2^SLACK: weights up to 2^SLACK are as exact in bf16 and fp32 as
+    // weights up to 1.  The slow loop moves it (and rescales) when a tile beats it by 2^8.
+    constexpr float SLACK = 64.0f;
+    auto sm_move_ref = [&](int c, float tmax) -> float {
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        float corr = 1.0f;
+        if (tmax > m_ref[c] + 8.0f) {
+            corr = __builtin_amdgcn_exp2f(m_ref[c] - tmax);              // first tile: exp2(-inf) = 0
+            m_ref[c] = tmax;
+            l_part[c] *= corr;
+        }
+        return corr;
+    };
+    // value MFMAs of one tile for both column blocks
+    auto values = [&](int tile, const u32x4 (&pw)[2][2], const u32x4 (&pl)[2][2]) {
+        const unsigned char *vb = &sm.v[tile & 1][0];
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ks2++) {
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][0] + db * (2 * PF_BLK)));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][1] + db * (2 * PF_BLK)));
+                typedef __attribute__((ext_vector_type(8))) short s16x8;
+                const bf16x8 va = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pw[c][ks2]), oacc[c][db], 0, 0, 0);
+                    if (precise)
+                        oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pl[c][ks2]), oacc[c][db], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // The accumulators live in AGPRs.  Written as ordinary arithmetic a rescale makes the
+    // compiler move them to VGPRs for the whole loop (and spill), and so does a rescale under a
+    // condition; so the fast loop has none, and the slow loop scales every tile, in place.
+    auto rescale = [&](const float (&corr)[2]) {
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int db = 0; db < 8; db++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    float tmp;
+                    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\t"
+                                 "v_accvgpr_write_b32 %0, %1"
+                                 : "+a"(oacc[c][db][i]), "=&v"(tmp)
+                                 : "v"(corr[c]));
+                }
+    };
+    // top of step t: K(t+1) and V(t) have landed (this wave's part, then everyone's; all reads of
+    // step t-1 are over as well), then the copies of K(t+2) and V(t+1) start
+    auto step_top = [&](int t) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PF_LDS_BARRIER();
+        if (t + 2 < n_tiles) issue(Kg, lds_k + (uint32_t)((t & 1) * PF_TILE), t + 2);
+        issue(Vg, lds_v + (uint32_t)(((t + 1) & 1) * PF_TILE), t + 1);
+    };
+
+    // ---- prologue: K(0), V(0), K(1); scores and softmax of tile 0 (sets the reference) ----
+    issue(Kg, lds_k, 0);
+    issue(Vg, lds_v, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PF_LDS_BARRIER();
+    if (n_tiles > 1) issue(Kg, lds_k + PF_TILE, 1);
+
+    u32x4 pw[2][2], pl[2][2];
+    {
+        f32x16 s[2];
+        scores(0, s);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            (void)sm_move_ref(c, sm_prep(0, c, s[c]));                  // nothing accumulated yet
+            sm_finish(c, s[c], pw[c], pl[c]);
+        }
+    }
+
+    // ---- fast loop: scores(t+1); softmax(t+1) beside values(t); no rescale ----
+    int t = 0;
+    bool slow = false;
+    for (; t + 1 < n_tiles; t++) {
+        step_top(t);
+        f32x16 s[2];
+        scores(t + 1, s);
+        u32x4 pwn[2][2], pln[2][2];
+        const float x0 = sm_prep(t + 1, 0, s[0]), x1 = sm_prep(t + 1, 1, s[1]);
+        if (__any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK)) {   // a row outgrew the reference
+            slow = true;
+            break;
+        }
+        sm_finish(0, s[0], pwn[0], pln[0]);
+        sm_finish(1, s[1], pwn[1], pln[1]);
+        values(t, pw, pl);
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int k2 = 0; k2 < 2; k2++) {
+                pw[c][k2] = pwn[c][k2];
+                pl[c][k2] = pln[c][k2];
+            }
+    }
+    // ---- slow loop (rare): the reference follows the maximum, accumulators rescaled every tile.
+    // It resumes step t after its top; the fast attempt only touched the scores (recomputed here).
+    if (slow) {
+        bool resumed = true;
+        for (; t + 1 < n_tiles; t++) {
+            if (!resumed) step_top(t);
+            resumed = false;
+            f32x16 s[2];
+            scores(t + 1, s);
+            u32x4 pwn[2][2], pln[2][2];
+            float corr[2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                corr[c] = sm_move_ref(c, sm_prep(t + 1, c, s[c]));
+                sm_finish(c, s[c], pwn[c], pln[c]);
+            }
+            values(t, pw, pl);
+            rescale(corr);
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int k2 = 0; k2 < 2; k2++) {
+                    pw[c][k2] = pwn[c][k2];
+                    pl[c][k2] = pln[c][k2];
+                }
+        }
+    }
+    // ---- last tile's values ----
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PF_LDS_BARRIER();
+    values(n_tiles - 1, pw, pl);
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const float l = l_part[c] + __shfl_xor(l_part[c], 32, 64);
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        if (row_live[c]) {
+            float *o = out + t_row[c] * q_stride + (size_t)(kvh * GROUP + j_row[c]) * PF_HD + 4 * g;
+#pragma unroll
+            for (int db = 0; db < 8; db++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++) {
+                    f32x4 w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) w[i] = oacc[c][db][4 * b4 + i] * inv;
+                    *(f32x4 *)(o + 32 * db + 8 * b4) = w;
+                }
+        }
     }
 }
 
@@ -252,17 +394,34 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     static bool attr_set = false;
     const size_t smem = sizeof(PfSmem);
     if (!attr_set) {
-        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP>,
+        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP, false>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP, true>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     constexpr int P = PF_ROWS / GROUP;
     const int64_t pblocks = (n + P - 1) / P;
     CWICK_REQUIRE(pblocks <= 0x7FFFFFFF && n_kv_heads <= 65535, "gqa_prefill: grid too large");
+    // Short prefixes: few keys carry the whole weight, so the 2^-9 rounding of each bf16 weight
+    // shows in an O(1) output.  Position blocks that see at most 2048 keys run the variant that
+    // also feeds the rounding residual through the matrix core (weights good to 2^-17).
+    int64_t n_prec = 0;
+    while (n_prec < pblocks) {
+        int64_t last_t = (n_prec + 1) * P - 1;
+        if (last_t > n - 1) last_t = n - 1;
+        if (pos0 + last_t + 1 > 2048) break;
+        n_prec++;
+    }
+    const float sl = scale * 1.44269504088896340736f;
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_PREFILL, s);
-        gqa_prefill_kernel<GROUP><<<dim3((unsigned)pblocks, n_kv_heads), PF_THREADS, smem, s>>>(
-            k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out);
+        if (pblocks > n_prec)
+            gqa_prefill_kernel<GROUP, false><<<dim3((unsigned)(pblocks - n_prec), n_kv_heads), PF_THREADS, smem, s>>>(
+                k, v, q, pos0, n, n_kv_heads, sl, out, n_prec);
+        if (n_prec > 0)
+            gqa_prefill_kernel<GROUP, true><<<dim3((unsigned)n_prec, n_kv_heads), PF_THREADS, smem, s>>>(
+                k, v, q, pos0, n, n_kv_heads, sl, out, 0);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
