@@ -64,14 +64,13 @@ struct PfSmem {
 #define PF_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 // PRECISE: the bf16 rounding residual of the weights goes through the matrix core as well
-// (position blocks that see at most 2048 keys; see the launcher).
+// (position blocks that see at most 2048 keys; see the launcher).  The body of one workgroup:
 template <int GROUP, bool PRECISE>
-__global__ void __launch_bounds__(PF_THREADS, 1)
-gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
-                   const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
-                   float scale_log2e, float *__restrict__ out, int64_t pblk_lo) {
+__device__ __forceinline__ void
+gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+                 const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
+                 float scale_log2e, float *__restrict__ out, int64_t pblk) {
     constexpr int P = PF_ROWS / GROUP;      // positions per workgroup
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     PfSmem &sm = *reinterpret_cast<PfSmem *>(smem_raw);
 
     const int tid = threadIdx.x;
@@ -81,8 +80,6 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     const int g = lane >> 5;                // 0/1
 
     const int kvh = blockIdx.y;
-    // heavy (late) position blocks first: better tail balance under the causal triangle
-    const int64_t pblk = pblk_lo + ((int64_t)gridDim.x - 1 - blockIdx.x);
     const int64_t t0 = pblk * P;
     const int n_heads = n_kv_heads * GROUP;
     const int64_t kv_stride = (int64_t)n_kv_heads * PF_HD;
@@ -126,16 +123,20 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     const uint16_t *Vg = V + (size_t)kvh * PF_HD + 8 * g;
     const uint32_t lds_k = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.k[0][0];
     const uint32_t lds_v = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.v[0][0];
-    auto issue = [&](const uint16_t *base, uint32_t lds_tile, int tile) {
+    auto copy_src = [&](const uint16_t *base, int tile) -> const uint16_t * {
         int64_t row = (int64_t)tile * PF_TK + cp_key;
         if (row > n_keys_all - 1) row = n_keys_all - 1;         // masked anyway
-        const uint16_t *src = base + row * kv_stride + 64 * wave;
+        return base + row * kv_stride + 64 * wave;
+    };
+    auto copy_one = [&](const uint16_t *src, uint32_t lds_tile, int i) {      // block 4 wave + i
+        const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK));
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     ::"v"(src + 16 * i), "s"(off) : "memory");
+    };
+    auto issue = [&](const uint16_t *base, uint32_t lds_tile, int tile) {
+        const uint16_t *src = copy_src(base, tile);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK));
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                         ::"v"(src + 16 * i), "s"(off) : "memory");
-        }
+        for (int i = 0; i < 4; i++) copy_one(src, lds_tile, i);
     };
 
     // K fragment of k-step ks: block ks, slot 32g + (l32 ^ 8g)
@@ -168,7 +169,9 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     // scores of one tile for both column blocks
     // One wave per SIMD: nothing hides an LDS round trip, so the fragments are fetched PF_PRE
     // k-steps ahead of the MFMAs that use them.
-    auto scores = [&](int tile, f32x16 (&s)[2]) {
+    // copy_t >= 0: the copies of K(copy_t + 2) and V(copy_t + 1) are issued between the MFMAs
+    // (an LDS-DMA instruction occupies the issue slot for about as long as two MFMAs run)
+    auto scores = [&](int tile, f32x16 (&s)[2], int copy_t) {
         const unsigned char *kb = &sm.k[tile & 1][0] + kfrag_off;
         const u32x4 *qb = &sm.qx[wave][0][lane];
         u32x4 ka[PF_PRE], qa[PF_PRE];
@@ -177,6 +180,11 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
             ka[ks] = *(const u32x4 *)(kb + ks * PF_BLK);
             if (ks >= PF_QX0) qa[ks] = qb[(ks - PF_QX0) * 64];
         }
+        const bool do_k = copy_t >= 0 && copy_t + 2 < n_tiles, do_v = copy_t >= 0;
+        const uint16_t *src_k = copy_src(Kg, do_k ? copy_t + 2 : 0);
+        const uint16_t *src_v = copy_src(Vg, do_v ? copy_t + 1 : 0);
+        const uint32_t dst_k = lds_k + (uint32_t)((copy_t & 1) * PF_TILE);
+        const uint32_t dst_v = lds_v + (uint32_t)(((copy_t + 1) & 1) * PF_TILE);
 #pragma unroll
         for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -191,6 +199,10 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
             }
             s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
             s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q1, s[1], 0, 0, 0);
+            if ((ks & 1) == 0) {
+                if (ks < 8) { if (do_k) copy_one(src_k, dst_k, ks >> 1); }
+                else if (do_v) copy_one(src_v, dst_v, (ks - 8) >> 1);
+            }
         }
     };
     // softmax bookkeeping of one tile and column block, in two parts.
@@ -250,20 +262,26 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     // value MFMAs of one tile for both column blocks
     auto values = [&](int tile, const u32x4 (&pw)[2][2], const u32x4 (&pl)[2][2]) {
         const unsigned char *vb = &sm.v[tile & 1][0];
+        // step st = 8 ks2 + db; its two transpose reads are issued PF_PRE steps ahead
+        s16x4 lo[PF_PRE], hi[PF_PRE];
+        auto fetch = [&](int st, int slot) {
+            const int ks2 = st >> 3, db = st & 7;
+            lo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][0] + db * (2 * PF_BLK)));
+            hi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][1] + db * (2 * PF_BLK)));
+        };
 #pragma unroll
-        for (int ks2 = 0; ks2 < 2; ks2++) {
+        for (int st = 0; st < PF_PRE; st++) fetch(st, st);
 #pragma unroll
-            for (int db = 0; db < 8; db++) {
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][0] + db * (2 * PF_BLK)));
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][1] + db * (2 * PF_BLK)));
-                typedef __attribute__((ext_vector_type(8))) short s16x8;
-                const bf16x8 va = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        for (int st = 0; st < 16; st++) {
+            const int ks2 = st >> 3, db = st & 7;
+            typedef __attribute__((ext_vector_type(8))) short s16x8;
+            const bf16x8 va = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo[st % PF_PRE], hi[st % PF_PRE], 0, 1, 2, 3, 4, 5, 6, 7));
+            if (st + PF_PRE < 16) fetch(st + PF_PRE, st % PF_PRE);
 #pragma unroll
-                for (int c = 0; c < 2; c++) {
-                    oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pw[c][ks2]), oacc[c][db], 0, 0, 0);
-                    if (precise)
-                        oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pl[c][ks2]), oacc[c][db], 0, 0, 0);
-                }
+            for (int c = 0; c < 2; c++) {
+                oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pw[c][ks2]), oacc[c][db], 0, 0, 0);
+                if (precise)
+                    oacc[c][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pl[c][ks2]), oacc[c][db], 0, 0, 0);
             }
         }
     };
@@ -285,12 +303,10 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
                 }
     };
     // top of step t: K(t+1) and V(t) have landed (this wave's part, then everyone's; all reads of
-    // step t-1 are over as well), then the copies of K(t+2) and V(t+1) start
-    auto step_top = [&](int t) {
+    // step t-1 are over as well, so the copies of K(t+2) and V(t+1) may start)
+    auto step_top = [&]() {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         PF_LDS_BARRIER();
-        if (t + 2 < n_tiles) issue(Kg, lds_k + (uint32_t)((t & 1) * PF_TILE), t + 2);
-        issue(Vg, lds_v + (uint32_t)(((t + 1) & 1) * PF_TILE), t + 1);
     };
 
     // ---- prologue: K(0), V(0), K(1); scores and softmax of tile 0 (sets the reference) ----
@@ -303,7 +319,7 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     u32x4 pw[2][2], pl[2][2];
     {
         f32x16 s[2];
-        scores(0, s);
+        scores(0, s, -1);
 #pragma unroll
         for (int c = 0; c < 2; c++) {
             (void)sm_move_ref(c, sm_prep(0, c, s[c]));                  // nothing accumulated yet
@@ -311,22 +327,26 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
         }
     }
 
-    // ---- fast loop: scores(t+1); softmax(t+1) beside values(t); no rescale ----
+    // ---- fast loop: scores(t+1); then softmax(t+1) beside values(t); no rescale.  The softmax
+    // is speculative: whether a row outgrew the reference is looked at after the MFMAs.
     int t = 0;
     bool slow = false;
     for (; t + 1 < n_tiles; t++) {
-        step_top(t);
+        step_top();
         f32x16 s[2];
-        scores(t + 1, s);
+        scores(t + 1, s, t);
         u32x4 pwn[2][2], pln[2][2];
+        const float l_save[2] = {l_part[0], l_part[1]};
         const float x0 = sm_prep(t + 1, 0, s[0]), x1 = sm_prep(t + 1, 1, s[1]);
-        if (__any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK)) {   // a row outgrew the reference
-            slow = true;
-            break;
-        }
         sm_finish(0, s[0], pwn[0], pln[0]);
         sm_finish(1, s[1], pwn[1], pln[1]);
         values(t, pw, pl);
+        if (__any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK)) {   // a row outgrew the reference
+            l_part[0] = l_save[0];
+            l_part[1] = l_save[1];
+            slow = true;
+            break;
+        }
 #pragma unroll
         for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -336,14 +356,13 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
             }
     }
     // ---- slow loop (rare): the reference follows the maximum, accumulators rescaled every tile.
-    // It resumes step t after its top; the fast attempt only touched the scores (recomputed here).
+    // It resumes step t after its top, copies and values(t); the scores are recomputed.
     if (slow) {
         bool resumed = true;
         for (; t + 1 < n_tiles; t++) {
-            if (!resumed) step_top(t);
-            resumed = false;
+            if (!resumed) step_top();
             f32x16 s[2];
-            scores(t + 1, s);
+            scores(t + 1, s, resumed ? -1 : t);
             u32x4 pwn[2][2], pln[2][2];
             float corr[2];
 #pragma unroll
@@ -351,7 +370,8 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
                 corr[c] = sm_move_ref(c, sm_prep(t + 1, c, s[c]));
                 sm_finish(c, s[c], pwn[c], pln[c]);
             }
-            values(t, pw, pl);
+            if (!resumed) values(t, pw, pl);
+            resumed = false;
             rescale(corr);
 #pragma unroll
             for (int c = 0; c < 2; c++)
@@ -387,6 +407,19 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     }
 }
 
+// One launch: position blocks below n_prec take the PRECISE body.
+template <int GROUP>
+__global__ void __launch_bounds__(PF_THREADS, 1)
+gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+                   const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
+                   float scale_log2e, float *__restrict__ out, int64_t n_prec) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    // heavy (late) position blocks first: better tail balance under the causal triangle
+    const int64_t pblk = (int64_t)gridDim.x - 1 - blockIdx.x;
+    if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk);
+    else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk);
+}
+
 template <int GROUP>
 static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
                            int n_kv_heads, const uint16_t *q, float scale, float *out,
@@ -394,9 +427,7 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     static bool attr_set = false;
     const size_t smem = sizeof(PfSmem);
     if (!attr_set) {
-        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP, false>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP, true>,
+        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
@@ -413,15 +444,10 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
         if (pos0 + last_t + 1 > 2048) break;
         n_prec++;
     }
-    const float sl = scale * 1.44269504088896340736f;
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_PREFILL, s);
-        if (pblocks > n_prec)
-            gqa_prefill_kernel<GROUP, false><<<dim3((unsigned)(pblocks - n_prec), n_kv_heads), PF_THREADS, smem, s>>>(
-                k, v, q, pos0, n, n_kv_heads, sl, out, n_prec);
-        if (n_prec > 0)
-            gqa_prefill_kernel<GROUP, true><<<dim3((unsigned)n_prec, n_kv_heads), PF_THREADS, smem, s>>>(
-                k, v, q, pos0, n, n_kv_heads, sl, out, 0);
+        gqa_prefill_kernel<GROUP><<<dim3((unsigned)pblocks, n_kv_heads), PF_THREADS, smem, s>>>(
+            k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

@@ -87,6 +87,27 @@ def test_gqa_prefill(hip, orc, pos0, n, nh, nkv):
     cache.free()
 
 
+def test_gqa_prefill_growing_scores(hip, orc):
+    """Scores that climb by far more than 2^64 along the keys: the rows must leave the fixed
+    softmax reference of their first tile and follow the maximum (rescaling path)."""
+    say("[case] gqa_prefill growing scores")
+    n, nh, nkv = 300, 16, 4
+    c = synth.cfg2_gqa_prefill(n, nh, nkv, 256, 0, seed=777)
+    k = synth.bf16_to_f32(c["k"]).reshape(n, nkv, 256)
+    q = synth.bf16_to_f32(c["q"]).reshape(n, nh, 256)
+    # a common direction whose weight grows with the key index: q.k gains about i * 4 per key
+    k[:, :, 0] = np.arange(n, dtype=np.float32)[:, None] * 0.5
+    q[:, :, 0] = 8.0 * 16.0                                   # times scale 1/16 -> 8 * 0.5 * i
+    ck = synth.f32_to_bf16(k.reshape(n, -1)); cq = synth.f32_to_bf16(q.reshape(n, nh, 256))
+    cache = hip.KVCache(n, nkv, 256)
+    cache.write(0, ck, c["v"].reshape(n, -1))
+    got = hip.gqa_prefill(cache, 0, cq, c["scale"])
+    ref = orc.gqa_prefill(cq, ck.reshape(n, nkv, 256), c["v"], 0, c["scale"], nthreads=0)
+    assert np.isfinite(got).all()
+    assert_close(got, ref, "gqa_prefill growing scores", strict=False)
+    cache.free()
+
+
 def test_gqa_prefill_declines_unsupported(hip):
     say("[case] gqa_prefill declines")
     cache = hip.KVCache(64, 4, 128)                       # head_dim 128: decode only
