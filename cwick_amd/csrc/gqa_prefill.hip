@@ -69,7 +69,7 @@ template <int GROUP, bool PRECISE>
 __device__ __forceinline__ void
 gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
                  const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
-                 float scale_log2e, float *__restrict__ out, int64_t pblk) {
+                 float scale_log2e, float *__restrict__ out, int64_t pblk, int kvh) {
     constexpr int P = PF_ROWS / GROUP;      // positions per workgroup
     PfSmem &sm = *reinterpret_cast<PfSmem *>(smem_raw);
 
@@ -79,7 +79,6 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     const int l32 = lane & 31;
     const int g = lane >> 5;                // 0/1
 
-    const int kvh = blockIdx.y;
     const int64_t t0 = pblk * P;
     const int n_heads = n_kv_heads * GROUP;
     const int64_t kv_stride = (int64_t)n_kv_heads * PF_HD;
@@ -414,10 +413,13 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
                    const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
                    float scale_log2e, float *__restrict__ out, int64_t n_prec) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    // heavy (late) position blocks first: better tail balance under the causal triangle
-    const int64_t pblk = (int64_t)gridDim.x - 1 - blockIdx.x;
-    if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk);
-    else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk);
+    // heavy (late) position blocks first, over all kv heads: workgroups are handed out in grid
+    // order, and under the causal triangle the last ones to start must be the short ones
+    const int64_t pblocks = (int64_t)gridDim.x / n_kv_heads;
+    const int64_t pblk = pblocks - 1 - (int64_t)blockIdx.x / n_kv_heads;
+    const int kvh = (int)(blockIdx.x % n_kv_heads);
+    if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
+    else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
 }
 
 template <int GROUP>
@@ -433,7 +435,7 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     }
     constexpr int P = PF_ROWS / GROUP;
     const int64_t pblocks = (n + P - 1) / P;
-    CWICK_REQUIRE(pblocks <= 0x7FFFFFFF && n_kv_heads <= 65535, "gqa_prefill: grid too large");
+    CWICK_REQUIRE(pblocks * n_kv_heads <= 0x7FFFFFFF, "gqa_prefill: grid too large");
     // Short prefixes: few keys carry the whole weight, so the 2^-9 rounding of each bf16 weight
     // shows in an O(1) output.  Position blocks that see at most 2048 keys run the variant that
     // also feeds the rounding residual through the matrix core (weights good to 2^-17).
@@ -446,7 +448,7 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     }
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_PREFILL, s);
-        gqa_prefill_kernel<GROUP><<<dim3((unsigned)pblocks, n_kv_heads), PF_THREADS, smem, s>>>(
+        gqa_prefill_kernel<GROUP><<<dim3((unsigned)(pblocks * n_kv_heads)), PF_THREADS, smem, s>>>(
             k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec);
     }
     CWICK_HIP_CALL(hipGetLastError());
