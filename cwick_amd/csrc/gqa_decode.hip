@@ -20,6 +20,8 @@
 #include "common.hpp"
 #include "merge.hpp"
 
+#include <cstdlib>
+
 namespace cwick {
 
 constexpr int GQA_DEC_THREADS = 256;
@@ -197,7 +199,10 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     constexpr int LPK = HD / 8, NGRP = GQA_DEC_THREADS / LPK;
     constexpr int step = NGRP * GQA_DEC_KB;   // rows one workgroup consumes per iteration
     // enough workgroups for ~2 per CU, each at least one full step
-    int64_t want = (int64_t)2 * num_cus() / n_kv_heads;
+    const char *env = getenv("CWICK_HIP_GQA_WG_PER_CU");
+    int per_cu = env ? atoi(env) : 2;
+    if (per_cu < 1 || per_cu > 8) per_cu = 2;
+    int64_t want = (int64_t)per_cu * num_cus() / n_kv_heads;
     if (want < 1) want = 1;
     if (want > MERGE_MAX_SPLITS) want = MERGE_MAX_SPLITS;
     int64_t per = (n_keys + want - 1) / want;
@@ -217,7 +222,8 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     CWICK_HIP_CALL(hipGetLastError());
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_DECODE_MERGE, s);
-        splitk_merge_kernel<HD><<<dim3(n_heads, 1), 256, 0, s>>>(part_acc, part_ml, n_splits, n_heads, out);
+        splitk_merge_wide_kernel<HD><<<dim3(n_heads, 1), 64 * (n_splits < 16 ? n_splits : 16), 0, s>>>(
+            part_acc, part_ml, n_splits, n_heads, out);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
