@@ -13,8 +13,13 @@
 //   2. one ordered pass emits every index with key > T and the first r indices
 //      with key == T, in ascending index order, through a block-wide scan.
 //
-// One workgroup of 1024 threads per batch row; the row (n * 4 bytes) is read
-// five times from L2.  Rows past min(k, n) are filled with -1.
+// One workgroup of 1024 threads per batch row.  Rows of up to 65536 scores (the
+// indexer's case) are read once: every thread keeps its 64 consecutive keys in
+// registers for all five passes, the first histogram pass counts into one of 32
+// lane-indexed copies (scores cluster in a few exponent buckets, and same-address
+// LDS atomics serialise), and the ordered emit places elements with ballots
+// inside a wave and one pass over the wave totals.  Longer rows take the streaming kernel,
+// which reads the row five times from L2.  Rows past min(k, n) are filled with -1.
 #include "common.hpp"
 
 namespace cwick {
@@ -159,6 +164,133 @@ topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     }
 }
 
+// ---- rows that fit the register file: n <= TOPK_THREADS * TOPK_EPT ----
+// Wave w owns the consecutive elements [w * 64 * ept, (w + 1) * 64 * ept); inside it lane l
+// holds elements base + 64 j + l, so the loads are coalesced and index order is (j, lane):
+// positions inside a wave come from ballots, positions of the waves from one block scan.
+constexpr int TOPK_EPT = 64;                   // keys per thread
+
+__global__ void __launch_bounds__(TOPK_THREADS)
+topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
+                      int32_t *__restrict__ out) {
+    // first pass: 32 copies of the histogram, one per lane (mod 32): scores cluster in a few
+    // exponent buckets and same-address LDS atomics of one instruction serialise
+    __shared__ uint32_t hist32[256 * 32];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t sh_gt[TOPK_WAVES], sh_eq[TOPK_WAVES];
+    __shared__ uint32_t sh_prefix, sh_remaining;
+    const float *sc = scores + (size_t)blockIdx.x * n;
+    int32_t *dst = out + (size_t)blockIdx.x * k;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t kk = k < n ? k : n;
+    for (int64_t i = kk + tid; i < k; i += TOPK_THREADS) dst[i] = -1;
+
+    const int ept = (int)((n + TOPK_THREADS - 1) / TOPK_THREADS);     // <= 64
+    const int64_t wbase = (int64_t)wave * 64 * ept;
+    // this lane holds elements j < jv
+    int64_t left = n - wbase - lane;
+    const int jv = left <= 0 ? 0 : (int)((left + 63) / 64 < ept ? (left + 63) / 64 : ept);
+    uint32_t key[TOPK_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_EPT; j++) key[j] = j < jv ? topk_key(sc[wbase + 64 * j + lane]) : 0u;
+    if (tid == 0) {
+        sh_prefix = 0u;
+        sh_remaining = (uint32_t)kk;
+    }
+    // ---- 1. find the key of the kk-th best element ----
+    uint32_t prefix = 0u, mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0u;
+        if (shift == 24) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) hist32[tid + TOPK_THREADS * c] = 0u;
+        }
+        __syncthreads();
+        if (shift == 24) {
+#pragma unroll
+            for (int j = 0; j < TOPK_EPT; j++)
+                if (j < jv) atomicAdd(&hist32[(key[j] >> 24) * 32 + (lane & 31)], 1u);
+            __syncthreads();
+            if (tid < 256) {
+                uint32_t c = 0u;
+#pragma unroll
+                for (int i = 0; i < 32; i++) c += hist32[tid * 32 + ((i + tid) & 31)];
+                hist[tid] = c;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TOPK_EPT; j++)
+                if (j < jv && (key[j] & mask) == prefix) atomicAdd(&hist[(key[j] >> shift) & 0xFFu], 1u);
+        }
+        __syncthreads();
+        if (tid < 64) {
+            // walk the 256 buckets from the largest digit down; lane b owns
+            // buckets 255-4b .. 252-4b
+            const uint32_t remaining = sh_remaining;
+            uint32_t c[4], sum = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                c[j] = hist[255 - (tid * 4 + j)];
+                sum += c[j];
+            }
+            uint32_t inc = sum;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                uint32_t t = __shfl_up(inc, o, 64);
+                if (tid >= o) inc += t;
+            }
+            uint32_t before = inc - sum;   // elements in strictly larger buckets
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (before < remaining && remaining <= before + c[j]) {
+                    sh_prefix = prefix | ((uint32_t)(255 - (tid * 4 + j)) << shift);
+                    sh_remaining = remaining - before;
+                }
+                before += c[j];
+            }
+        }
+        __syncthreads();
+        prefix = sh_prefix;
+        mask |= 0xFFu << shift;
+    }
+    const uint32_t T = prefix;
+    const uint32_t r = sh_remaining;       // elements equal to T that belong to the selection
+
+    // ---- 2. ordered emit ----
+    uint32_t w_gt = 0u, w_eq = 0u;         // wave totals (uniform)
+#pragma unroll
+    for (int j = 0; j < TOPK_EPT; j++) {
+        w_gt += (uint32_t)__builtin_popcountll(__ballot(j < jv && key[j] > T));
+        w_eq += (uint32_t)__builtin_popcountll(__ballot(j < jv && key[j] == T));
+    }
+    if (lane == 0) {
+        sh_gt[wave] = w_gt;
+        sh_eq[wave] = w_eq;
+    }
+    __syncthreads();
+    uint32_t eq_before = 0u, pos = 0u;     // ties / outputs of the waves before this one
+    for (int w = 0; w < wave; w++) {
+        const uint32_t e = sh_eq[w];
+        const uint32_t take_e = eq_before >= r ? 0u : (r - eq_before < e ? r - eq_before : e);
+        pos += sh_gt[w] + take_e;
+        eq_before += e;
+    }
+    const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int j = 0; j < TOPK_EPT; j++) {
+        const bool gt = j < jv && key[j] > T;
+        const bool eq = j < jv && key[j] == T;
+        const uint64_t m_eq = __ballot(eq);
+        const uint32_t my_eq_rank = eq_before + (uint32_t)__builtin_popcountll(m_eq & lt);
+        const bool take = gt || (eq && my_eq_rank < r);
+        const uint64_t m_take = __ballot(take);
+        if (take) dst[pos + (uint32_t)__builtin_popcountll(m_take & lt)] = (int32_t)(wbase + 64 * j + lane);
+        pos += (uint32_t)__builtin_popcountll(m_take);
+        eq_before += (uint32_t)__builtin_popcountll(m_eq);
+    }
+}
+
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s) {
     CWICK_REQUIRE(scores && out_idx, "topk: null pointer");
@@ -167,7 +299,10 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
     {
         ProfScope ps(CWICK_HIP_PROF_TOPK, s);
-        topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)
+            topk_radix_reg_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        else
+            topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
