@@ -128,7 +128,7 @@ def bench_cfg3(hip, synth, T, stream):
     wall, kern = T.run(step)
     alg = 32768 * (576 + 20) + 128 * 576 * 2 + 128 * 512 * 4
     flops = 2 * 128 * 32768 * (576 + 512)
-    t = kern["mla_fwd_kernel"]["avg_us"] * 1e-6
+    t = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
     return {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
                         "+ 5 fp32 block scales/token, bf16 q",
             "us_per_step": wall * 1e6, "kernels": kern, "alg_bytes": alg, "flops": flops,
@@ -148,7 +148,7 @@ def bench_cfg4(hip, synth, T, stream):
     wall, kern = T.run(step)
     keys = c["n"] * c["pos0"] + c["n"] * (c["n"] + 1) // 2
     flops = 2 * c["nh"] * (576 + 512) * keys
-    t = kern["mla_fwd_kernel"]["avg_us"] * 1e-6
+    t = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
     return {"workload": "cfg4 MLA chunked prefill, 4096 queries appended to 28672 FP8 latent rows",
             "us_per_step": wall * 1e6, "kernels": kern, "flops": flops,
             "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
@@ -173,7 +173,7 @@ def bench_cfg5(hip, synth, T, stream):
     idx_bytes = B * N * 132
     idx_flops = B * 2 * c["ih"] * N * 128
     t_idx = kern["indexer_scores_kernel"]["avg_us"] * 1e-6
-    t_mla = kern["mla_fwd_kernel"]["avg_us"] * 1e-6
+    t_mla = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
     mla_flops = B * 2 * 128 * K * 1088
     return {"workload": "cfg5 DSA decode, 8 independent queries (own caches): indexer 64x128 over "
                         "65536 FP8 keys -> exact top-2048 -> sparse MLA",
