@@ -129,10 +129,14 @@ def bench_cfg3(hip, synth, T, stream):
     alg = 32768 * (576 + 20) + 128 * 576 * 2 + 128 * 512 * 4
     flops = 2 * 128 * 32768 * (576 + 512)
     t = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
+    # HBM bytes of one launch of mla_dsplit_kernel at this geometry (64 key slices): FETCH_SIZE and
+    # WRITE_SIZE of rocprofv3 --pmc, each scaled by what a 256 MiB copy reads on the same counter
+    # (profiles/mla_decode_cfg3_pmc_traffic.txt): 20.90 MB read + 16.84 MB of split-K partials written
+    traffic = 20413 * 1024 + 16448 * 1024
     return {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
                         "+ 5 fp32 block scales/token, bf16 q",
             "us_per_step": wall * 1e6, "kernels": kern, "alg_bytes": alg, "flops": flops,
-            "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s"),
+            "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s", traffic),
             "roofline_mfma": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
             "wall_GBps": alg / wall / 1e9}, (c, out)
 
@@ -216,6 +220,9 @@ def main():
                     help="which configurations to time besides the headline (cfg4 takes ~1 min)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (a kernel of known HBM traffic, "
+                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
     if a.gpus != 1:
         log("bench.py: this build shows one GPU's share of the path; --gpus %d is not run "
@@ -232,6 +239,14 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
     wanted = {int(x) for x in a.configs.split(",") if x} | {3}
+
+    if a.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     results = {}
     # headline first: exactly K steps of cfg3
