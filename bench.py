@@ -128,8 +128,8 @@ def bench_cfg3(hip, synth, T, stream):
     wall, kern = T.run(step)
     alg = 32768 * (576 + 20) + 128 * 576 * 2 + 128 * 512 * 4
     flops = 2 * 128 * 32768 * (576 + 512)
-    t = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
-    # HBM bytes of one launch of mla_dsplit_kernel at this geometry (64 key slices): FETCH_SIZE and
+    t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
+    # HBM bytes of one launch of mla_roles_kernel at this geometry (64 key slices): FETCH_SIZE and
     # WRITE_SIZE of rocprofv3 --pmc, each scaled by what a 256 MiB copy reads on the same counter
     # (profiles/mla_decode_cfg3_pmc_traffic.txt): 20.90 MB read + 16.84 MB of split-K partials written
     traffic = 20413 * 1024 + 16448 * 1024
@@ -152,7 +152,7 @@ def bench_cfg4(hip, synth, T, stream):
     wall, kern = T.run(step)
     keys = c["n"] * c["pos0"] + c["n"] * (c["n"] + 1) // 2
     flops = 2 * c["nh"] * (576 + 512) * keys
-    t = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
+    t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
     return {"workload": "cfg4 MLA chunked prefill, 4096 queries appended to 28672 FP8 latent rows",
             "us_per_step": wall * 1e6, "kernels": kern, "flops": flops,
             "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
@@ -177,7 +177,7 @@ def bench_cfg5(hip, synth, T, stream):
     idx_bytes = B * N * 132
     idx_flops = B * 2 * c["ih"] * N * 128
     t_idx = kern["indexer_scores_kernel"]["avg_us"] * 1e-6
-    t_mla = kern["mla_dsplit_kernel"]["avg_us"] * 1e-6
+    t_mla = kern["mla_roles_kernel"]["avg_us"] * 1e-6
     mla_flops = B * 2 * 128 * K * 1088
     return {"workload": "cfg5 DSA decode, 8 independent queries (own caches): indexer 64x128 over "
                         "65536 FP8 keys -> exact top-2048 -> sparse MLA",

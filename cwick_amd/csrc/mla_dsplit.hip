@@ -1,8 +1,8 @@
 // mla_dsplit.hip -- absorbed-latent MLA with the contraction split over the waves
 // (decode, sparse decode and chunked prefill of src/attention.c:749-811 /
-// :1010-1019 over the FP8 latent).  This is the kernel the entry points use;
-// mla_stream.hip and mla.hip are earlier schedules kept selectable
-// (CWICK_HIP_MLA=stream|v1) as comparison arms.
+// :1010-1019 over the FP8 latent).  An earlier schedule than the one the entry
+// points use (mla_roles.hip), kept selectable as a comparison arm
+// (CWICK_HIP_MLA=dsplit).
 //
 //   workgroup = 8 waves = 2 teams of 4, 32 query rows (heads of one query) x one
 //   key slice; the teams take alternate 32-key tiles of the slice and meet once,
@@ -42,19 +42,6 @@
 #include <cstring>
 
 namespace cwick {
-int launch_mla_decode_v1(const uint8_t *rows, const float *scales, int64_t row_bstride,
-                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                         hipStream_t s);
-int launch_mla_prefill_v1(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
-                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
-int launch_mla_decode_v2(const uint8_t *rows, const float *scales, int64_t row_bstride,
-                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                         hipStream_t s);
-int launch_mla_prefill_v2(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
-                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
-
 namespace {
 
 constexpr int KDIM = CWICK_HIP_LATENT_KDIM;   // 576
@@ -583,16 +570,6 @@ int run(Params &p, hipStream_t s) {
     return 1;
 }
 
-// CWICK_HIP_MLA = v1 | stream selects an earlier schedule (comparison arms)
-int variant() {
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("CWICK_HIP_MLA");
-        v = !e ? 0 : (!strcmp(e, "v1") ? 1 : (!strcmp(e, "stream") ? 2 : 0));
-    }
-    return v;
-}
-
 int splits_per_cu() {
     static int v = -1;
     if (v < 0) {
@@ -605,16 +582,10 @@ int splits_per_cu() {
 
 }  // namespace
 
-int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
+int launch_mla_decode_v3(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
                       int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
                       hipStream_t s) {
-    if (variant() == 1)
-        return launch_mla_decode_v1(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
-                                    q, n_heads, scale, out, s);
-    if (variant() == 2)
-        return launch_mla_decode_v2(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
-                                    q, n_heads, scale, out, s);
     CWICK_REQUIRE(rows && scales && q && out, "mla_decode: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 4096, "mla_decode: batch %d", batch);
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
@@ -644,10 +615,8 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
     return run(p, s);
 }
 
-int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+int launch_mla_prefill_v3(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
                        const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s) {
-    if (variant() == 1) return launch_mla_prefill_v1(rows, scales, pos0, n, q, n_heads, scale, out, s);
-    if (variant() == 2) return launch_mla_prefill_v2(rows, scales, pos0, n, q, n_heads, scale, out, s);
     CWICK_REQUIRE(rows && scales && q && out, "mla_prefill: null pointer");
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill: n_heads %d (1..128)", n_heads);
     CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= ((int64_t)1 << 31) - 1 && n <= (1 << 22),

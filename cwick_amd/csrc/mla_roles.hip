@@ -1,0 +1,754 @@
+// mla_roles.hip -- absorbed-latent MLA over the FP8 latent (decode, sparse decode and chunked
+// prefill of src/attention.c:749-811 / :1010-1019).  This is the kernel the entry points use;
+// mla_dsplit.hip, mla_stream.hip and mla.hip are earlier schedules kept selectable
+// (CWICK_HIP_MLA=dsplit|stream|v1) as comparison arms.
+//
+//   workgroup = 12 waves, 32 query rows (heads of one query) x one key slice, walked in tiles
+//   of 64 keys.  The waves take one of two roles:
+//     waves 0..7  score: wave (kb, hh) takes keys 16 kb..+15 of the tile and heads 16 hh..+15:
+//                 S^T = K Q^T on v_mfma_scale_f32_16x16x128_f8f6f4 with K as stored (E4M3) and Q
+//                 as two E4M3 terms with a shared E8M0 scale per head and 128-dim block; the five
+//                 block products are combined with the keys' fp32 block scales, exponentiated
+//                 against the wave's reference m, and published through LDS as fp16 value weights
+//                 exp2(s - m) * scale[key][block] * 2^(10 - e), one copy per scale block, already in
+//                 the fragment order of the value MFMA, together with m and e (a power of two
+//                 above every scale seen so far, so that the weights fit fp16);
+//     waves 8..11 accumulate: wave cw owns output dims 128 cw..+127 (one scale block) for all 32
+//                 heads: O^T += V^T W^T on v_mfma_f32_16x16x32_f16, V^T read transposed from the
+//                 tile (ds_read_b64_tr_b8) and widened E4M3 -> fp16 (exact).
+//   The roles are one tile apart (tile t+1 is scored while tile t is accumulated), so a step has
+//   a single workgroup barrier and nobody waits for an exchange inside it.  The softmax
+//   reference is lazy: a scoring wave keeps the reference every wave knows (m_ref) unless its own
+//   tile exceeds it by 2^LAZY; the m it used travels with the weights, and the accumulating
+//   waves (and the scorers, for their sums) bring everything to the common maximum one step
+//   later -- almost always a comparison and nothing else.  Each scoring lane keeps the sum of
+//   its own keys; the sums meet once, after the loop.
+//   Tiles are copied global -> LDS by global_load_lds (no registers), three stages: tile t+2 is
+//   fetched during step t.  The copies are issued from inline assembly and the barrier waits for
+//   LDS traffic only, so the compiler never makes anything wait for the tile in flight.
+//
+//   LDS tile layout [16-byte column][key 0..63][16 B]: the K fragment is two 16-byte reads per
+//   lane, 256 B contiguous per 16 keys; the V^T fragment of 32 keys x 16 dims is one
+//   ds_read_b64_tr_b8, 128 B contiguous per 16-lane group (keys 8 g..8 g+7 of the half).
+//
+//   Split-K partials are stored per 16 heads in accumulator-fragment order
+//   [split][16-head block][dim block][lane][4] (every store 1 KiB contiguous);
+//   mla_merge_frag16_kernel reads them in the same order with all loads in flight.
+#include "common.hpp"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace cwick {
+int launch_mla_decode_v1(const uint8_t *rows, const float *scales, int64_t row_bstride,
+                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
+                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
+                         hipStream_t s);
+int launch_mla_prefill_v1(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+int launch_mla_decode_v2(const uint8_t *rows, const float *scales, int64_t row_bstride,
+                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
+                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
+                         hipStream_t s);
+int launch_mla_prefill_v2(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+int launch_mla_decode_v3(const uint8_t *rows, const float *scales, int64_t row_bstride,
+                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
+                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
+                         hipStream_t s);
+int launch_mla_prefill_v3(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+
+namespace {
+
+constexpr int KDIM = CWICK_HIP_LATENT_KDIM;   // 576
+constexpr int VDIM = CWICK_HIP_LATENT_VDIM;   // 512
+constexpr int NBLK = CWICK_HIP_LATENT_NBLK;   // 5
+constexpr int THREADS = 768;                  // waves 0..7 score, waves 8..11 accumulate values
+constexpr int TK = 64;                        // keys per tile
+constexpr int HB = 16;                        // heads per head half (partials are laid out per 16 heads)
+constexpr int HW = 32;                        // heads per workgroup
+constexpr int NST = 3;                        // tile stages
+constexpr int NCOL = KDIM / 16;               // 36 sixteen-byte columns per row
+constexpr int NDB = VDIM / 16;                // 32 sixteen-dim output blocks
+constexpr float LAZY = 4.0f;                  // the reference moves when a tile exceeds it by 2^LAZY
+constexpr int WEXP = 10;                      // fp16 weights are p * scale * 2^(WEXP - e), scale < 2^e
+constexpr int E_NONE = -1000;                 // no scale seen yet
+constexpr int MERGE_MAX_SPLITS = 1024;
+
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+typedef __attribute__((address_space(3))) void lds_void;
+
+struct Params {
+    const uint8_t *rows;
+    const float *scales;
+    int64_t row_bstride, scale_bstride, n_rows;
+    const int32_t *sel;
+    int64_t n_list, list_step;
+    const uint16_t *q;
+    int nh, nq;
+    float scale;
+    int n_splits;
+    int64_t keys_per_split;   // multiple of TK
+    float *out, *part_acc, *part_ml;
+};
+
+struct Tile {
+    uint8_t kv[NCOL][TK][16];     // [16-byte column][key][16]     36864 B
+    float sc[NBLK][TK];           // [block][key]                   1280 B
+};
+struct Xch {                       // what the scoring waves publish per tile
+    // fp16 value weights exp2(s - m) * scale[key][block] * 2^(WEXP - e), laid out as the B
+    // fragments of the value MFMA: [scale block][head half][32-key half][slot group g][head n]
+    // [4 dwords]; contraction slot 8 g + j of a half is key 8 g + j of that half
+    uint32_t w[4][2][2][4][16][4];
+    float m[2][16][4];            // [head half][head][key block]: the reference m the weights are relative to
+    int e[2][4];                  // [head half][key block]: ... and the exponent e
+};
+struct Smem {
+    Tile tile[NST];
+    Xch x[2];
+};
+// Q of one (head half, 128-dim block) in MFMA operand order, dword-interleaved by lane; for the
+// rope block `hi` is the combined hi|lo register set
+struct QPark { int hi[8][64]; int lo[8][64]; int sc[64]; };
+static_assert(10 * sizeof(QPark) <= sizeof(Tile) + 2 * sizeof(Xch), "Q park area");
+
+__device__ __forceinline__ float pow2i(int e) {
+    e = e > 126 ? 126 : (e < -126 ? -126 : e);
+    return __builtin_bit_cast(float, (uint32_t)(e + 127) << 23);
+}
+
+// both fp16 halves of a dword times f
+__device__ __forceinline__ uint32_t scale_f16x2(uint32_t x, float f) {
+    const _Float16 h = (_Float16)f;
+    const f16x2 r = __builtin_bit_cast(f16x2, x) * (f16x2){h, h};
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+#define LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+__global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool scorer = wave < 8;
+    const int kb = wave & 3;         // scoring role: keys 16 kb .. 16 kb + 15 of the tile
+    const int hh = (wave >> 2) & 1;  //               heads 16 hh .. 16 hh + 15
+    const int cw = wave & 3;         // value role: dims 128 cw .. +127 = scale block cw
+    const int vblk = cw;
+    const int n = lane & 15;         // head column / key row of a 16-block / dim row
+    const int g = lane >> 4;         // 32-wide contraction block (QK) / 8-wide (PV)
+
+    const int n_hb = (p.nh + HW - 1) / HW;
+    const int64_t total = (int64_t)gridDim.x;
+    int64_t unit = blockIdx.x;
+    if (total % 8 == 0) unit = (unit % 8) * (total / 8) + unit / 8;
+    const int hb = (int)(unit % n_hb);
+    const int split = (int)((unit / n_hb) % p.n_splits);
+    int y = (int)(unit / ((int64_t)n_hb * p.n_splits));
+    if (p.list_step > 0) y = p.nq - 1 - y;          // causal prefill: the queries with the most keys start first
+
+    const uint8_t *rows = p.rows + (size_t)y * p.row_bstride;
+    const float *scales = p.scales + (size_t)y * p.scale_bstride;
+    const int32_t *sel = p.sel ? p.sel + (size_t)y * p.n_list : nullptr;
+    const int64_t limit = p.n_list + (int64_t)y * p.list_step;
+    const int64_t k_begin = (int64_t)split * p.keys_per_split;
+    int64_t k_end = k_begin + p.keys_per_split;
+    if (k_end > limit) k_end = limit;
+    const int n_tiles = k_end > k_begin ? (int)((k_end - k_begin + TK - 1) / TK) : 0;
+
+    // copy role: lane = key of the tile
+    auto row_of = [&](int t) -> int {
+        const int64_t i = k_begin + (int64_t)t * TK + lane;
+        int64_t r = -1;
+        if (t < n_tiles && i < k_end) {
+            r = sel ? (int64_t)sel[i] : i;
+            if (r < 0 || r >= p.n_rows) r = -1;
+        }
+        return (int)r;
+    };
+    // global -> LDS copies in assembly: the compiler keeps no account of them, so nothing in the
+    // loop waits for the tile in flight except the s_waitcnt before the barrier
+    auto dma16 = [&](const void *gp, const void *lp) {
+        const uint32_t off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void *)lp);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gp), "s"(off) : "memory");
+    };
+    auto dma4 = [&](const void *gp, const void *lp) {
+        const uint32_t off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void *)lp);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gp), "s"(off) : "memory");
+    };
+    // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; wave w copies pieces w, w+12, w+24, w+36
+    auto issue = [&](int r, Tile *b) {
+        const int64_t rc = r >= 0 ? r : 0;            // masked positions fetch row 0, weight 0
+        const uint8_t *gsrc = rows + rc * KDIM + 16 * wave;
+        dma16(gsrc, &b->kv[wave][0][0]);
+        dma16(gsrc + 192, &b->kv[wave + 12][0][0]);
+        dma16(gsrc + 384, &b->kv[wave + 24][0][0]);
+        if (wave < 5) dma4(scales + rc * NBLK + wave, &b->sc[wave][0]);
+    };
+
+    int row0 = row_of(0), row1 = row_of(1);
+    uint64_t valid_nxt = __ballot(row0 >= 0);          // of the tile the next scoring step reads
+    uint64_t valid_aft = __ballot(row1 >= 0);
+    if (n_tiles > 0) issue(row0, &sm.tile[0]);
+    if (n_tiles > 1) issue(row1, &sm.tile[1]);
+
+    // ---- Q for 2 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
+    // 128-dim block (the hardware pairs the scale of lane (n, g) with k-elements that live in other
+    // lanes of the same head, so the four lanes must agree; both terms use it).
+    // lane (n, g) holds head n of the half, dims 128 b + 32 g + [0, 32); the rope block is one
+    // register set: lanes g < 2 hold the hi term of dims 512 + 32 g.., lanes g >= 2 the lo term of
+    // dims 512 + 32 (g - 2).. (the key side repeats its bytes).  Unit u = 5 hhu + b is prepared
+    // by wave u and parked in the third tile stage and the exchange area (neither in use yet).
+    {
+        QPark *park = reinterpret_cast<QPark *>(&sm.tile[2]);
+        if (wave < 10) {
+            const int u = wave;
+            const int hhu = u / 5, b = u % 5;
+            int head = hb * HW + 16 * hhu + n;
+            if (head >= p.nh) head = p.nh - 1;
+            const uint16_t *qrow = p.q + ((size_t)y * p.nh + head) * KDIM;
+            const uint16_t *src = qrow + (b < 4 ? 128 * b + 32 * g : 512 + 32 * (g & 1));
+            float qv[32];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const u32x4 w = *(const u32x4 *)(src + 8 * c);
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    qv[8 * c + 2 * d] = bf16lo_to_f32(w[d]);
+                    qv[8 * c + 2 * d + 1] = bf16hi_to_f32(w[d]);
+                }
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; j++) amax = fmaxf(amax, __builtin_fabsf(qv[j]));
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            int s = amax > 0.0f ? (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu) - 127 - 7 : 0;
+            s = s < -110 ? -110 : s;
+            const float inv = pow2i(-s), mul = pow2i(s);
+            QPark *qp = park + u;
+            const bool rope_lo = b == 4 && g >= 2;
+#pragma unroll
+            for (int d = 0; d < 8; d++) {
+                int wh = 0, wl = 0;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; h2++) {
+                    const float a0 = qv[4 * d + 2 * h2], a1 = qv[4 * d + 2 * h2 + 1];
+                    if (h2 == 0) wh = __builtin_amdgcn_cvt_pk_fp8_f32(a0 * inv, a1 * inv, wh, false);
+                    else wh = __builtin_amdgcn_cvt_pk_fp8_f32(a0 * inv, a1 * inv, wh, true);
+                    const f32x2 back = h2 == 0 ? __builtin_amdgcn_cvt_pk_f32_fp8(wh, false) : __builtin_amdgcn_cvt_pk_f32_fp8(wh, true);
+                    const float r0 = a0 - back[0] * mul, r1 = a1 - back[1] * mul;
+                    if (h2 == 0) wl = __builtin_amdgcn_cvt_pk_fp8_f32(r0 * inv, r1 * inv, wl, false);
+                    else wl = __builtin_amdgcn_cvt_pk_fp8_f32(r0 * inv, r1 * inv, wl, true);
+                }
+                qp->hi[d][lane] = rope_lo ? wl : wh;
+                qp->lo[d][lane] = wl;
+            }
+            qp->sc[lane] = 127 + s;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tiles 0 and 1 have landed (this wave's share)
+        LDS_BARRIER();
+    }
+
+    const float c0 = p.scale * 1.44269504088896340736f;   // scores in log2 units
+    float m_ref[2] = {-INFINITY, -INFINITY};          // of head 16 h2 + n; every wave tracks the same values
+    int e_ref = E_NONE;                               // ... and the same exponent above every scale seen so far
+    float l_priv = 0.0f, l_pend = 0.0f;               // scoring role: sum over this lane's keys (head 16 hh + n), relative to m_ref / to the tile's m_loc
+
+    // transpose-read addressing for V^T: lane i of 16-lane group g supplies key kappa(g, i>>1),
+    // bytes 8 (i & 1) .. +7 of the sixteen-byte column
+    const int tr_key = 8 * g + (n >> 1);
+    const int tr_off = (8 * cw) * (TK * 16) + tr_key * 16 + 8 * (n & 1);
+
+    if (scorer) {
+        i32x8 qhi[4], qlo[4], qrope;
+        int qsc0 = 0, qsc1 = 0;                           // scale bytes of blocks 0..3 / of the rope block
+        QPark *park = reinterpret_cast<QPark *>(&sm.tile[2]);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const QPark *qp = park + 5 * hh + b;
+#pragma unroll
+            for (int d = 0; d < 8; d++) {
+                qhi[b][d] = qp->hi[d][lane];
+                qlo[b][d] = qp->lo[d][lane];
+            }
+            qsc0 |= qp->sc[lane] << (8 * b);
+        }
+        const QPark *qp = park + 5 * hh + 4;
+#pragma unroll
+        for (int d = 0; d < 8; d++) qrope[d] = qp->hi[d][lane];
+        qsc1 = qp->sc[lane];
+
+        LDS_BARRIER();                                // before copies or weights land in the park area
+        // step t: waves 0..7 score tile t+1 (if any), waves 8..11 accumulate tile t (if any).
+        // Nothing the compiler has in flight may cross into the loop: its waits would also wait
+        // for the copies.
+        asm volatile("" : "+v"(qhi[0]), "+v"(qhi[1]), "+v"(qhi[2]), "+v"(qhi[3]), "+v"(qlo[0]), "+v"(qlo[1]), "+v"(qlo[2]), "+v"(qlo[3]), "+v"(qrope), "+v"(qsc0), "+v"(qsc1));
+#pragma clang loop unroll(disable)
+        for (int t = -1; t < n_tiles; t++) {
+            if (t >= 0 && t + 2 < n_tiles) {
+                const int r2 = row_of(t + 2);
+                issue(r2, &sm.tile[(t + 2) % NST]);       // the stage tile t-1 left at the last barrier
+                valid_aft = __ballot(r2 >= 0);
+            }
+            if (t >= 0) {
+                // what the four key blocks of tile t used as reference for this half's heads
+                const f32x4 ml = *(const f32x4 *)&sm.x[t & 1].m[hh][n][0];
+                const i32x4 el = *(const i32x4 *)&sm.x[t & 1].e[hh][0];
+                const int e01 = el[0] > el[1] ? el[0] : el[1], e23 = el[2] > el[3] ? el[2] : el[3];
+                const int e_t = e01 > e23 ? e01 : e23;
+                e_ref = e_t > e_ref ? e_t : e_ref;    // the sums do not carry the exponent
+                const float mr = hh ? m_ref[1] : m_ref[0];
+                const float m_new = fmaxf(mr, fmaxf(fmaxf(ml[0], ml[1]), fmaxf(ml[2], ml[3])));
+                if (__any(m_new != mr || ml[0] != m_new || ml[1] != m_new || ml[2] != m_new || ml[3] != m_new)) {
+                    const float mo = kb == 0 ? ml[0] : kb == 1 ? ml[1] : kb == 2 ? ml[2] : ml[3];
+                    const float fo = mo == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mo - m_new);
+                    const float c = mr == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mr - m_new);
+                    l_priv = l_priv * c + fo * l_pend;
+                    if (hh) m_ref[1] = m_new; else m_ref[0] = m_new;
+                } else {
+                    l_priv += l_pend;
+                }
+            }
+            if (t + 1 < n_tiles) {
+                // ---- scores S^T[key][head] for keys 16 kb.., heads 16 hh.. of tile t+1 ----
+                const Tile &T = sm.tile[(t + 1) % NST];
+                Xch &X = sm.x[(t + 1) & 1];
+                const uint64_t valid = valid_nxt;
+                auto kfrag = [&](int b) -> i32x8 {
+                    const int col = b < 4 ? 8 * b + 2 * g : 32 + 2 * (g & 1);
+                    const u32x4 k0 = *(const u32x4 *)&T.kv[col][16 * kb + n][0];
+                    const u32x4 k1 = *(const u32x4 *)&T.kv[col + 1][16 * kb + n][0];
+                    return (i32x8){(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
+                };
+                const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                f32x4 S = z4;
+                f32x4 scw[4];
+                i32x8 kA = kfrag(0);
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const i32x8 kN = kfrag(b + 1);
+                    scw[b] = *(const f32x4 *)&T.sc[b][16 * kb + 4 * g];
+                    const f32x4 scb = scw[b];
+                    f32x4 acc;
+                    if (b == 0) {
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
+                    } else if (b == 1) {
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 1, qsc0);
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 1, qsc0);
+                    } else if (b == 2) {
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 2, qsc0);
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 2, qsc0);
+                    } else {
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
+                        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
+                    }
+                    S += acc * scb;
+                    kA = kN;
+                }
+                {
+                    const f32x4 scb = *(const f32x4 *)&T.sc[4][16 * kb + 4 * g];
+                    const f32x4 acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qrope, z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc1);
+                    S += acc * scb;
+                }
+                S *= c0;
+                if (valid != ~0ull) {
+                    const uint32_t bits = (uint32_t)(valid >> (16 * kb)) >> (4 * g);
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (!((bits >> i) & 1u)) S[i] = -INFINITY;
+                }
+                float lmax = fmaxf(fmaxf(S[0], S[1]), fmaxf(S[2], S[3]));
+                const float mr = hh ? m_ref[1] : m_ref[0];
+                float m_loc = mr;
+                if (__any(lmax > mr + LAZY)) {            // rare after the first tiles: only then the lanes of a head confer
+                    lmax = fmaxf(lmax, __shfl_xor(lmax, 16, 64));
+                    lmax = fmaxf(lmax, __shfl_xor(lmax, 32, 64));
+                    m_loc = lmax > mr + LAZY ? lmax : mr;
+                }
+                const float m_use = m_loc == -INFINITY ? 0.0f : m_loc;
+                f32x4 P;
+#pragma unroll
+                for (int i = 0; i < 4; i++) P[i] = __builtin_amdgcn_exp2f(S[i] - m_use);
+                l_pend = (P[0] + P[1]) + (P[2] + P[3]);   // of this lane's four keys, relative to m_loc
+                // normaliser of the fp16 weights: a power of two above every scale of the tile's keys
+                // (of all four value blocks); it only grows, and only then the lanes confer
+                int e_loc = e_ref;
+                {
+                    float smax = fmaxf(fmaxf(fmaxf(scw[0][0], scw[0][1]), fmaxf(scw[0][2], scw[0][3])),
+                                       fmaxf(fmaxf(scw[1][0], scw[1][1]), fmaxf(scw[1][2], scw[1][3])));
+                    smax = fmaxf(smax, fmaxf(fmaxf(fmaxf(scw[2][0], scw[2][1]), fmaxf(scw[2][2], scw[2][3])),
+                                             fmaxf(fmaxf(scw[3][0], scw[3][1]), fmaxf(scw[3][2], scw[3][3]))));
+                    const float thr = e_ref == E_NONE ? 0.0f : pow2i(e_ref);   // scales below 2^e_ref fit
+                    if (__any(smax >= thr && smax > 0.0f)) {
+#pragma unroll
+                        for (int o = 32; o > 0; o >>= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
+                        const int e_tile = (int)((__builtin_bit_cast(uint32_t, smax) >> 23) & 0xFFu) - 126;
+                        e_loc = e_tile > e_ref ? e_tile : e_ref;
+                    }
+                }
+                const float wfac = e_loc == E_NONE ? 0.0f : pow2i(WEXP - e_loc);
+#pragma unroll
+                for (int i = 0; i < 4; i++) P[i] *= wfac;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const f32x4 wv = P * scw[b];
+                    u32x2 d;
+                    d[0] = pack_f16_rne(wv[0], wv[1]);
+                    d[1] = pack_f16_rne(wv[2], wv[3]);
+                    *(u32x2 *)&X.w[b][hh][kb >> 1][2 * (kb & 1) + (g >> 1)][n][2 * (g & 1)] = d;   // keys 16 (kb & 1) + 4 g + i of the half
+                }
+                if (g == 0) X.m[hh][n][kb] = m_loc;
+                if (lane == 0) X.e[hh][kb] = e_loc;
+            }
+            valid_nxt = valid_aft;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of tile t+2 has landed
+            LDS_BARRIER();
+        }
+
+        // ---- the sums of the scoring role meet in LDS (the exchange area is free now) ----
+        float *lsum = reinterpret_cast<float *>(&sm.x[0]);            // [head half][head][key block]
+        float ls = l_priv + __shfl_xor(l_priv, 16, 64);
+        ls += __shfl_xor(ls, 32, 64);
+        if (g == 0) lsum[(hh * 16 + n) * 4 + kb] = ls;
+        LDS_BARRIER();
+    } else {
+        LDS_BARRIER();                                // before copies or weights land in the park area
+        f32x4 oacc[2][8];                                 // [head half][dim block]: dims 128 cw + 16 j + 4 g + i, head n
+#pragma unroll
+        for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) oacc[h2][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        asm volatile("" ::: "memory");
+#pragma clang loop unroll(disable)
+        for (int t = -1; t < n_tiles; t++) {
+            if (t >= 0 && t + 2 < n_tiles) {
+                const int r2 = row_of(t + 2);
+                issue(r2, &sm.tile[(t + 2) % NST]);       // the stage tile t-1 left at the last barrier
+                valid_aft = __ballot(r2 >= 0);
+            }
+            if (t >= 0) {
+                // ---- values O^T[dim][head] += V^T P^T for dims 128 cw.., all 32 heads, tile t ----
+                const Tile &T = sm.tile[t % NST];
+                const Xch &X = sm.x[t & 1];
+                const uint8_t *vbase = &T.kv[0][0][0] + tr_off;
+                u32x4 pw[2][2];                           // [head half][key half]
+                f32x4 ml[2];
+#pragma unroll
+                for (int h2 = 0; h2 < 2; h2++) {
+#pragma unroll
+                    for (int kh = 0; kh < 2; kh++) pw[h2][kh] = *(const u32x4 *)&X.w[vblk][h2][kh][g][n][0];
+                    ml[h2] = *(const f32x4 *)&X.m[h2][n][0];
+                }
+                // the exponents the key blocks used (the two head halves agree: same keys, same rule)
+                const i32x4 el = *(const i32x4 *)&X.e[0][0];
+                const int e01 = el[0] > el[1] ? el[0] : el[1], e23 = el[2] > el[3] ? el[2] : el[3];
+                const int e_t = e01 > e23 ? e01 : e23;
+                const int e_new = e_t > e_ref ? e_t : e_ref;
+                const bool e_moved = e_new != e_ref || el[0] != e_new || el[1] != e_new || el[2] != e_new || el[3] != e_new;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; h2++) {
+                    const float m_new = fmaxf(m_ref[h2], fmaxf(fmaxf(ml[h2][0], ml[h2][1]), fmaxf(ml[h2][2], ml[h2][3])));
+                    if (e_moved || __any(m_new != m_ref[h2] || ml[h2][0] != m_new || ml[h2][1] != m_new || ml[h2][2] != m_new || ml[h2][3] != m_new)) {
+                        float f[4];
+#pragma unroll
+                        for (int k = 0; k < 4; k++)
+                            f[k] = (ml[h2][k] == -INFINITY || el[k] == E_NONE) ? 0.0f : __builtin_amdgcn_exp2f(ml[h2][k] - m_new) * pow2i(el[k] - e_new);
+                        const float c = (m_ref[h2] == -INFINITY || e_ref == E_NONE) ? 1.0f : __builtin_amdgcn_exp2f(m_ref[h2] - m_new) * pow2i(e_ref - e_new);
+                        m_ref[h2] = m_new;
+#pragma unroll
+                        for (int j = 0; j < 8; j++) oacc[h2][j] *= c;
+                        // weights were taken relative to each key block's own reference: bring them to m_new
+                        // (slot group g of half kh holds keys of key block 2 kh + g / 2)
+                        const float fsel0 = (g >> 1) ? f[1] : f[0], fsel1 = (g >> 1) ? f[3] : f[2];
+#pragma unroll
+                        for (int kh = 0; kh < 2; kh++)
+#pragma unroll
+                            for (int d = 0; d < 4; d++) {
+                                const float fk = kh ? fsel1 : fsel0;
+                                pw[h2][kh][d] = scale_f16x2(pw[h2][kh][d], fk);
+                            }
+                    }
+                }
+                e_ref = e_new;
+#pragma unroll
+                for (int j0 = 0; j0 < 8; j0 += 4) {
+                    i32x2 vt[4][2];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int kh = 0; kh < 2; kh++)
+                            vt[j][kh] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(vbase + (j0 + j) * (TK * 16) + kh * (32 * 16)));
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int kh = 0; kh < 2; kh++) {
+                            u32x4 vh;
+                            vh[0] = e4m3x2_to_f16x2<false>((uint32_t)vt[j][kh][0]);
+                            vh[1] = e4m3x2_to_f16x2<true>((uint32_t)vt[j][kh][0]);
+                            vh[2] = e4m3x2_to_f16x2<false>((uint32_t)vt[j][kh][1]);
+                            vh[3] = e4m3x2_to_f16x2<true>((uint32_t)vt[j][kh][1]);
+                            const f16x8 va = __builtin_bit_cast(f16x8, vh);
+                            oacc[0][j0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(f16x8, pw[0][kh]), oacc[0][j0 + j], 0, 0, 0);
+                            oacc[1][j0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(f16x8, pw[1][kh]), oacc[1][j0 + j], 0, 0, 0);
+                        }
+                }
+            }
+            valid_nxt = valid_aft;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of tile t+2 has landed
+            LDS_BARRIER();
+        }
+
+        const float *lsum = reinterpret_cast<const float *>(&sm.x[0]);
+        LDS_BARRIER();
+        // ---- every value wave owns its dims: write the partial (or the result) directly ----
+#pragma unroll
+        for (int h2 = 0; h2 < 2; h2++) {
+            const f32x4 lv = *(const f32x4 *)&lsum[(h2 * 16 + n) * 4];
+            const float L = (lv[0] + lv[1]) + (lv[2] + lv[3]);
+            const int head = hb * HW + 16 * h2 + n;
+            if (head >= p.nh) continue;
+            const float unit_f = e_ref == E_NONE ? 0.0f : pow2i(e_ref - WEXP);   // the accumulators are in units of 2^(e_ref - WEXP)
+            const float fin = p.n_splits == 1 ? (L > 0.0f ? unit_f / L : 0.0f) : unit_f;
+            const size_t pb = ((size_t)y * p.n_splits + split) * (2 * n_hb) + 2 * hb + h2;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int db = 8 * cw + j;
+                const f32x4 v = oacc[h2][j] * fin;
+                // accumulator register i <-> dim 16 db + 4 g + i
+                if (p.n_splits == 1) *(f32x4 *)(p.out + ((size_t)y * p.nh + head) * VDIM + 16 * db + 4 * g) = v;
+                else *(f32x4 *)(p.part_acc + pb * (HB * VDIM) + ((size_t)db * 64 + lane) * 4) = v;   // [db][lane][4]
+            }
+            if (p.n_splits > 1 && cw == 0 && g == 0) {
+                p.part_ml[(pb * HB + n) * 2 + 0] = m_ref[h2] * 0.69314718055994530942f;
+                p.part_ml[(pb * HB + n) * 2 + 1] = L;
+            }
+        }
+    }
+}
+
+// merge of fragment-layout partials [y][split][16-head block][dim block][lane][4]: workgroup =
+// one dim block of one 16-head block; its waves (up to sixteen, one per split when there are
+// fewer) take splits w, w + n_waves, ... and meet in LDS.  Every wave has all its loads in
+// flight at once (eight splits per batch); which splits exist is uniform per wave, so absent
+// ones cost nothing.
+constexpr int MW = 16;
+__global__ void __launch_bounds__(64 * MW)
+mla_merge_frag16_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
+                        int n_splits, int n_hb16, int nh, float *__restrict__ out) {
+    __shared__ float red_m[MW][64];
+    __shared__ float red_l[MW][64];
+    __shared__ f32x4 red_a[MW][64];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), mw = (int)blockDim.x >> 6;
+    const int db = blockIdx.x % NDB, hb = blockIdx.x / NDB, y = blockIdx.y;
+    const int n = lane & 15, g = lane >> 4;
+    const size_t sb = (size_t)y * n_splits;
+    const float *ml = part_ml + ((sb * n_hb16 + hb) * HB + n) * 2;
+    const size_t ml_stride = (size_t)n_hb16 * HB * 2;
+    const float *pa = part_acc + (sb * n_hb16 + hb) * (HB * VDIM) + ((size_t)db * 64 + lane) * 4;
+    const size_t pa_stride = (size_t)n_hb16 * HB * VDIM;
+
+    // first batch: everything in flight before anything is waited for
+    f32x4 a0[8];
+    f32x2 v0[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int s = wv + mw * j;
+        v0[j] = (f32x2){-INFINITY, 0.0f};
+        a0[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        if (s < n_splits) {
+            v0[j] = *(const f32x2 *)(ml + s * ml_stride);
+            a0[j] = *(const f32x4 *)(pa + s * pa_stride);
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; j++) mx = fmaxf(mx, v0[j][0]);
+    for (int s = wv + 8 * mw; s < n_splits; s += mw) mx = fmaxf(mx, ml[s * ml_stride]);
+    red_m[wv][lane] = mx;
+    __syncthreads();
+    for (int w = 0; w < mw; w++) mx = fmaxf(mx, red_m[w][lane]);
+
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float ls = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float c = v0[j][0] == -INFINITY ? 0.0f : __expf(v0[j][0] - mx);
+        ls = __builtin_fmaf(v0[j][1], c, ls);
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(a0[j][r], c, acc[r]);
+    }
+    for (int s0 = wv + 8 * mw; s0 < n_splits; s0 += 8 * mw) {
+        f32x4 a[8];
+        f32x2 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int s = s0 + mw * j;
+            v[j] = (f32x2){-INFINITY, 0.0f};
+            a[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            if (s < n_splits) {
+                v[j] = *(const f32x2 *)(ml + s * ml_stride);
+                a[j] = *(const f32x4 *)(pa + s * pa_stride);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float c = v[j][0] == -INFINITY ? 0.0f : __expf(v[j][0] - mx);
+            ls = __builtin_fmaf(v[j][1], c, ls);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(a[j][r], c, acc[r]);
+        }
+    }
+    red_l[wv][lane] = ls;
+    red_a[wv][lane] = acc;
+    __syncthreads();
+    if (wv != 0) return;
+    float l = 0.f;
+    f32x4 r4 = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < mw; w++) {
+        l += red_l[w][lane];
+        const f32x4 t = red_a[w][lane];
+#pragma unroll
+        for (int r = 0; r < 4; r++) r4[r] += t[r];
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const int head = hb * HB + n;
+    if (head >= nh) return;
+#pragma unroll
+    for (int r = 0; r < 4; r++) r4[r] *= inv;
+    // accumulator register i <-> dim 16 db + 4 g + i
+    *(f32x4 *)(out + ((size_t)y * nh + head) * VDIM + 16 * db + 4 * g) = r4;
+}
+
+int run(Params &p, hipStream_t s) {
+    static bool attr_set = false;
+    const size_t smem = sizeof(Smem);
+    if (!attr_set) {
+        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)mla_roles_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    const int n_hb = (p.nh + HW - 1) / HW;
+    const int64_t total = (int64_t)n_hb * p.n_splits * p.nq;
+    CWICK_REQUIRE(total <= 0x7FFFFFFF, "mla: grid of %lld workgroups is too large", (long long)total);
+    if (p.n_splits > 1) {
+        const size_t acc_b = (size_t)p.nq * p.n_splits * n_hb * HW * VDIM * sizeof(float);
+        const size_t ml_b = (size_t)p.nq * p.n_splits * n_hb * HW * 2 * sizeof(float);
+        char *ws = (char *)workspace(s, acc_b + ml_b);
+        CWICK_REQUIRE(ws, "mla: workspace allocation failed");
+        p.part_acc = (float *)ws;
+        p.part_ml = (float *)(ws + acc_b);
+    }
+    {
+        ProfScope ps(CWICK_HIP_PROF_MLA, s);
+        mla_roles_kernel<<<dim3((unsigned)total), THREADS, smem, s>>>(p);
+    }
+    CWICK_HIP_CALL(hipGetLastError());
+    if (p.n_splits > 1) {
+        ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
+        mla_merge_frag16_kernel<<<dim3(2 * n_hb * NDB, p.nq), 64 * (p.n_splits < MW ? p.n_splits : MW), 0, s>>>(
+            p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out);
+        CWICK_HIP_CALL(hipGetLastError());
+    }
+    return 1;
+}
+
+// CWICK_HIP_MLA = v1 | stream | dsplit selects an earlier schedule (comparison arms)
+int variant() {
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("CWICK_HIP_MLA");
+        v = !e ? 0 : (!strcmp(e, "v1") ? 1 : (!strcmp(e, "stream") ? 2 : (!strcmp(e, "dsplit") ? 3 : 0)));
+    }
+    return v;
+}
+
+int splits_per_cu() {
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("CWICK_HIP_MLA_WG_PER_CU");
+        v = e ? atoi(e) : 1;
+        if (v < 1 || v > 8) v = 1;
+    }
+    return v;
+}
+
+}  // namespace
+
+int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
+                      int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
+                      int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
+                      hipStream_t s) {
+    if (variant() == 1)
+        return launch_mla_decode_v1(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
+                                    q, n_heads, scale, out, s);
+    if (variant() == 2)
+        return launch_mla_decode_v2(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
+                                    q, n_heads, scale, out, s);
+    if (variant() == 3)
+        return launch_mla_decode_v3(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
+                                    q, n_heads, scale, out, s);
+    CWICK_REQUIRE(rows && scales && q && out, "mla_decode: null pointer");
+    CWICK_REQUIRE(batch >= 1 && batch <= 4096, "mla_decode: batch %d", batch);
+    CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
+    CWICK_REQUIRE(n_rows >= 1 && n_rows <= ((int64_t)1 << 31) - 1, "mla_decode: n_rows %lld",
+                  (long long)n_rows);
+    CWICK_REQUIRE(n_list >= 1 && n_list <= ((int64_t)1 << 31) - 1, "mla_decode: n_list %lld",
+                  (long long)n_list);
+    CWICK_REQUIRE(sel || n_list <= n_rows, "mla_decode: n_list %lld exceeds n_rows %lld",
+                  (long long)n_list, (long long)n_rows);
+    CWICK_REQUIRE(scale > 0.0f && scale < INFINITY, "mla_decode: scale must be positive");
+    CWICK_REQUIRE((uintptr_t)rows % 16 == 0 && row_bstride % 16 == 0 && (uintptr_t)q % 16 == 0 &&
+                      (uintptr_t)out % 16 == 0 && (uintptr_t)scales % 4 == 0,
+                  "mla_decode: rows, q and out must be 16-byte aligned");
+    Params p{};
+    p.rows = rows; p.scales = scales; p.row_bstride = row_bstride; p.scale_bstride = scale_bstride;
+    p.n_rows = n_rows; p.sel = sel; p.n_list = n_list; p.list_step = 0;
+    p.q = q; p.nh = n_heads; p.nq = batch; p.scale = scale; p.out = out;
+    // one workgroup is resident per CU: one round of workgroups
+    const int n_hb = (n_heads + HW - 1) / HW;
+    int64_t want = (int64_t)splits_per_cu() * num_cus() / ((int64_t)n_hb * batch);
+    if (want < 1) want = 1;
+    if (want > MERGE_MAX_SPLITS) want = MERGE_MAX_SPLITS;
+    int64_t per = (n_list + want - 1) / want;
+    per = ((per + TK - 1) / TK) * TK;
+    p.keys_per_split = per;
+    p.n_splits = (int)((n_list + per - 1) / per);
+    return run(p, s);
+}
+
+int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
+                       const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s) {
+    if (variant() == 1) return launch_mla_prefill_v1(rows, scales, pos0, n, q, n_heads, scale, out, s);
+    if (variant() == 2) return launch_mla_prefill_v2(rows, scales, pos0, n, q, n_heads, scale, out, s);
+    if (variant() == 3) return launch_mla_prefill_v3(rows, scales, pos0, n, q, n_heads, scale, out, s);
+    CWICK_REQUIRE(rows && scales && q && out, "mla_prefill: null pointer");
+    CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill: n_heads %d (1..128)", n_heads);
+    CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= ((int64_t)1 << 31) - 1 && n <= (1 << 22),
+                  "mla_prefill: pos0 %lld n %lld", (long long)pos0, (long long)n);
+    CWICK_REQUIRE(scale > 0.0f && scale < INFINITY, "mla_prefill: scale must be positive");
+    CWICK_REQUIRE((uintptr_t)rows % 16 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)out % 16 == 0,
+                  "mla_prefill: rows, q and out must be 16-byte aligned");
+    Params p{};
+    p.rows = rows; p.scales = scales; p.row_bstride = 0; p.scale_bstride = 0;
+    p.n_rows = pos0 + n; p.sel = nullptr; p.n_list = pos0 + 1; p.list_step = 1;
+    p.q = q; p.nh = n_heads; p.nq = (int)n; p.scale = scale; p.out = out;
+    p.n_splits = 1;
+    p.keys_per_split = ((pos0 + n + TK - 1) / TK) * TK;
+    return run(p, s);
+}
+
+}  // namespace cwick

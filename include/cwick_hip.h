@@ -253,8 +253,8 @@ enum {
     CWICK_HIP_PROF_GQA_DECODE = 0,      /* gqa_decode_split_kernel */
     CWICK_HIP_PROF_GQA_DECODE_MERGE,    /* splitk_merge_wide_kernel<256|128> after it */
     CWICK_HIP_PROF_GQA_PREFILL,         /* gqa_prefill_kernel */
-    CWICK_HIP_PROF_MLA,                 /* mla_dsplit_kernel (decode, sparse, prefill) */
-    CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag_kernel after it */
+    CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill) */
+    CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag16_kernel after it */
     CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel */
     CWICK_HIP_PROF_TOPK,                /* topk_radix_reg_kernel / topk_radix_kernel */
     CWICK_HIP_PROF_COUNT
