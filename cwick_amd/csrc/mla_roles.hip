@@ -9,23 +9,27 @@
 //                 S^T = K Q^T on v_mfma_scale_f32_16x16x128_f8f6f4 with K as stored (E4M3) and Q
 //                 as two E4M3 terms with a shared E8M0 scale per head and 128-dim block; the five
 //                 block products are combined with the keys' fp32 block scales, exponentiated
-//                 against the wave's reference m, and published through LDS as fp16 value weights
-//                 exp2(s - m) * scale[key][block] * 2^(10 - e), one copy per scale block, already in
-//                 the fragment order of the value MFMA, together with m and e (a power of two
-//                 above every scale seen so far, so that the weights fit fp16);
+//                 against the wave's reference m, and published through LDS as fp16
+//                 probabilities exp2(s - m), already in the fragment order of the value MFMA,
+//                 together with m;
 //     waves 8..11 accumulate: wave cw owns output dims 128 cw..+127 (one scale block) for all 32
-//                 heads: O^T += V^T W^T on v_mfma_f32_16x16x32_f16, V^T read transposed from the
-//                 tile (ds_read_b64_tr_b8) and widened E4M3 -> fp16 (exact).
+//                 heads: it turns the probabilities into weights p * scale[key][cw] * 2^(10 - e)
+//                 (packed fp16 multiplies; 2^e is above every scale the wave has seen, so the
+//                 weights fit fp16) and runs O^T += V^T W^T on v_mfma_f32_16x16x32_f16, V^T read
+//                 transposed from the tile (ds_read_b64_tr_b8) and widened E4M3 -> fp16 (exact).
 //   The roles are one tile apart (tile t+1 is scored while tile t is accumulated), so a step has
 //   a single workgroup barrier and nobody waits for an exchange inside it.  The softmax
 //   reference is lazy: a scoring wave keeps the reference every wave knows (m_ref) unless its own
-//   tile exceeds it by 2^LAZY; the m it used travels with the weights, and the accumulating
-//   waves (and the scorers, for their sums) bring everything to the common maximum one step
-//   later -- almost always a comparison and nothing else.  Each scoring lane keeps the sum of
-//   its own keys; the sums meet once, after the loop.
-//   Tiles are copied global -> LDS by global_load_lds (no registers), three stages: tile t+2 is
-//   fetched during step t.  The copies are issued from inline assembly and the barrier waits for
-//   LDS traffic only, so the compiler never makes anything wait for the tile in flight.
+//   tile exceeds it by 2^LAZY; the m it used travels with the probabilities, and the
+//   accumulating waves (and the scorers, for their sums) bring everything to the common maximum
+//   one step later -- almost always a comparison and nothing else.  Each scoring lane keeps the
+//   sum of its own keys; the sums meet once, after the loop.
+//   Tiles are copied global -> LDS by global_load_lds (no registers) into four stages: tile t+3
+//   is fetched during step t, two tiles ahead of its first use.  In the loop only the value
+//   waves issue copies: a wave that issues them stalls while the memory pipeline takes them, and
+//   the scoring waves are the long pole of a step.  The copies are issued from inline assembly
+//   and the barrier waits for LDS traffic only, so the compiler never makes anything wait for
+//   the tiles in flight.
 //
 //   LDS tile layout [16-byte column][key 0..63][16 B]: the K fragment is two 16-byte reads per
 //   lane, 256 B contiguous per 16 keys; the V^T fragment of 32 keys x 16 dims is one
@@ -68,7 +72,7 @@ constexpr int THREADS = 768;                  // waves 0..7 score, waves 8..11 a
 constexpr int TK = 64;                        // keys per tile
 constexpr int HB = 16;                        // heads per head half (partials are laid out per 16 heads)
 constexpr int HW = 32;                        // heads per workgroup
-constexpr int NST = 3;                        // tile stages
+constexpr int NST = 4;                        // tile stages
 constexpr int NCOL = KDIM / 16;               // 36 sixteen-byte columns per row
 constexpr int NDB = VDIM / 16;                // 32 sixteen-dim output blocks
 constexpr float LAZY = 4.0f;                  // the reference moves when a tile exceeds it by 2^LAZY
@@ -104,12 +108,11 @@ struct Tile {
     float sc[NBLK][TK];           // [block][key]                   1280 B
 };
 struct Xch {                       // what the scoring waves publish per tile
-    // fp16 value weights exp2(s - m) * scale[key][block] * 2^(WEXP - e), laid out as the B
-    // fragments of the value MFMA: [scale block][head half][32-key half][slot group g][head n]
-    // [4 dwords]; contraction slot 8 g + j of a half is key 8 g + j of that half
-    uint32_t w[4][2][2][4][16][4];
-    float m[2][16][4];            // [head half][head][key block]: the reference m the weights are relative to
-    int e[2][4];                  // [head half][key block]: ... and the exponent e
+    // fp16 probabilities exp2(s - m), laid out as the B fragments of the value MFMA:
+    // [head half][32-key half][slot group g][head n][4 dwords]; contraction slot 8 g + j of a
+    // half is key 8 g + j of that half
+    uint32_t p[2][2][4][16][4];
+    float m[2][16][4];            // [head half][head][key block]: the reference m they are relative to
 };
 struct Smem {
     Tile tile[NST];
@@ -119,6 +122,7 @@ struct Smem {
 // rope block `hi` is the combined hi|lo register set
 struct QPark { int hi[8][64]; int lo[8][64]; int sc[64]; };
 static_assert(10 * sizeof(QPark) <= sizeof(Tile) + 2 * sizeof(Xch), "Q park area");
+static_assert(sizeof(Tile) * NST + 2 * sizeof(Xch) <= 160 * 1024, "LDS");
 
 __device__ __forceinline__ float pow2i(int e) {
     e = e > 126 ? 126 : (e < -126 ? -126 : e);
@@ -129,6 +133,11 @@ __device__ __forceinline__ float pow2i(int e) {
 __device__ __forceinline__ uint32_t scale_f16x2(uint32_t x, float f) {
     const _Float16 h = (_Float16)f;
     const f16x2 r = __builtin_bit_cast(f16x2, x) * (f16x2){h, h};
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ uint32_t mul_f16x2(uint32_t a, uint32_t b) {
+    const f16x2 r = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
     return __builtin_bit_cast(uint32_t, r);
 }
 
@@ -197,11 +206,12 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         if (wave < 5) dma4(scales + rc * NBLK + wave, &b->sc[wave][0]);
     };
 
-    int row0 = row_of(0), row1 = row_of(1);
-    uint64_t valid_nxt = __ballot(row0 >= 0);          // of the tile the next scoring step reads
-    uint64_t valid_aft = __ballot(row1 >= 0);
-    if (n_tiles > 0) issue(row0, &sm.tile[0]);
-    if (n_tiles > 1) issue(row1, &sm.tile[1]);
+    {
+        const int row0 = row_of(0), row1 = row_of(1), row2 = row_of(2);
+        if (n_tiles > 0) issue(row0, &sm.tile[0]);
+        if (n_tiles > 1) issue(row1, &sm.tile[1]);
+        if (n_tiles > 2) issue(row2, &sm.tile[2]);
+    }
 
     // ---- Q for 2 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
     // 128-dim block (the hardware pairs the scale of lane (n, g) with k-elements that live in other
@@ -211,7 +221,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     // dims 512 + 32 (g - 2).. (the key side repeats its bytes).  Unit u = 5 hhu + b is prepared
     // by wave u and parked in the third tile stage and the exchange area (neither in use yet).
     {
-        QPark *park = reinterpret_cast<QPark *>(&sm.tile[2]);
+        QPark *park = reinterpret_cast<QPark *>(&sm.tile[NST - 1]);
         if (wave < 10) {
             const int u = wave;
             const int hhu = u / 5, b = u % 5;
@@ -257,13 +267,12 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             }
             qp->sc[lane] = 127 + s;
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tiles 0 and 1 have landed (this wave's share)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tiles 0, 1 and 2 have landed (this wave's share)
         LDS_BARRIER();
     }
 
     const float c0 = p.scale * 1.44269504088896340736f;   // scores in log2 units
     float m_ref[2] = {-INFINITY, -INFINITY};          // of head 16 h2 + n; every wave tracks the same values
-    int e_ref = E_NONE;                               // ... and the same exponent above every scale seen so far
     float l_priv = 0.0f, l_pend = 0.0f;               // scoring role: sum over this lane's keys (head 16 hh + n), relative to m_ref / to the tile's m_loc
 
     // transpose-read addressing for V^T: lane i of 16-lane group g supplies key kappa(g, i>>1),
@@ -274,7 +283,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     if (scorer) {
         i32x8 qhi[4], qlo[4], qrope;
         int qsc0 = 0, qsc1 = 0;                           // scale bytes of blocks 0..3 / of the rope block
-        QPark *park = reinterpret_cast<QPark *>(&sm.tile[2]);
+        QPark *park = reinterpret_cast<QPark *>(&sm.tile[NST - 1]);
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             const QPark *qp = park + 5 * hh + b;
@@ -295,20 +304,14 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         // Nothing the compiler has in flight may cross into the loop: its waits would also wait
         // for the copies.
         asm volatile("" : "+v"(qhi[0]), "+v"(qhi[1]), "+v"(qhi[2]), "+v"(qhi[3]), "+v"(qlo[0]), "+v"(qlo[1]), "+v"(qlo[2]), "+v"(qlo[3]), "+v"(qrope), "+v"(qsc0), "+v"(qsc1));
+        int row_nxt = row_of(0);
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
-            if (t >= 0 && t + 2 < n_tiles) {
-                const int r2 = row_of(t + 2);
-                issue(r2, &sm.tile[(t + 2) % NST]);       // the stage tile t-1 left at the last barrier
-                valid_aft = __ballot(r2 >= 0);
-            }
+            const int row_now = row_nxt;              // rows of tile t+1, fetched one step ahead
+            row_nxt = row_of(t + 2);
             if (t >= 0) {
                 // what the four key blocks of tile t used as reference for this half's heads
                 const f32x4 ml = *(const f32x4 *)&sm.x[t & 1].m[hh][n][0];
-                const i32x4 el = *(const i32x4 *)&sm.x[t & 1].e[hh][0];
-                const int e01 = el[0] > el[1] ? el[0] : el[1], e23 = el[2] > el[3] ? el[2] : el[3];
-                const int e_t = e01 > e23 ? e01 : e23;
-                e_ref = e_t > e_ref ? e_t : e_ref;    // the sums do not carry the exponent
                 const float mr = hh ? m_ref[1] : m_ref[0];
                 const float m_new = fmaxf(mr, fmaxf(fmaxf(ml[0], ml[1]), fmaxf(ml[2], ml[3])));
                 if (__any(m_new != mr || ml[0] != m_new || ml[1] != m_new || ml[2] != m_new || ml[3] != m_new)) {
@@ -325,7 +328,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 // ---- scores S^T[key][head] for keys 16 kb.., heads 16 hh.. of tile t+1 ----
                 const Tile &T = sm.tile[(t + 1) % NST];
                 Xch &X = sm.x[(t + 1) & 1];
-                const uint64_t valid = valid_nxt;
+                const uint64_t valid = __ballot(row_now >= 0);
                 auto kfrag = [&](int b) -> i32x8 {
                     const int col = b < 4 ? 8 * b + 2 * g : 32 + 2 * (g & 1);
                     const u32x4 k0 = *(const u32x4 *)&T.kv[col][16 * kb + n][0];
@@ -334,13 +337,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 };
                 const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
                 f32x4 S = z4;
-                f32x4 scw[4];
                 i32x8 kA = kfrag(0);
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     const i32x8 kN = kfrag(b + 1);
-                    scw[b] = *(const f32x4 *)&T.sc[b][16 * kb + 4 * g];
-                    const f32x4 scb = scw[b];
+                    const f32x4 scb = *(const f32x4 *)&T.sc[b][16 * kb + 4 * g];
                     f32x4 acc;
                     if (b == 0) {
                         acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
@@ -383,38 +384,14 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) P[i] = __builtin_amdgcn_exp2f(S[i] - m_use);
                 l_pend = (P[0] + P[1]) + (P[2] + P[3]);   // of this lane's four keys, relative to m_loc
-                // normaliser of the fp16 weights: a power of two above every scale of the tile's keys
-                // (of all four value blocks); it only grows, and only then the lanes confer
-                int e_loc = e_ref;
                 {
-                    float smax = fmaxf(fmaxf(fmaxf(scw[0][0], scw[0][1]), fmaxf(scw[0][2], scw[0][3])),
-                                       fmaxf(fmaxf(scw[1][0], scw[1][1]), fmaxf(scw[1][2], scw[1][3])));
-                    smax = fmaxf(smax, fmaxf(fmaxf(fmaxf(scw[2][0], scw[2][1]), fmaxf(scw[2][2], scw[2][3])),
-                                             fmaxf(fmaxf(scw[3][0], scw[3][1]), fmaxf(scw[3][2], scw[3][3]))));
-                    const float thr = e_ref == E_NONE ? 0.0f : pow2i(e_ref);   // scales below 2^e_ref fit
-                    if (__any(smax >= thr && smax > 0.0f)) {
-#pragma unroll
-                        for (int o = 32; o > 0; o >>= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
-                        const int e_tile = (int)((__builtin_bit_cast(uint32_t, smax) >> 23) & 0xFFu) - 126;
-                        e_loc = e_tile > e_ref ? e_tile : e_ref;
-                    }
-                }
-                const float wfac = e_loc == E_NONE ? 0.0f : pow2i(WEXP - e_loc);
-#pragma unroll
-                for (int i = 0; i < 4; i++) P[i] *= wfac;
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    const f32x4 wv = P * scw[b];
                     u32x2 d;
-                    d[0] = pack_f16_rne(wv[0], wv[1]);
-                    d[1] = pack_f16_rne(wv[2], wv[3]);
-                    *(u32x2 *)&X.w[b][hh][kb >> 1][2 * (kb & 1) + (g >> 1)][n][2 * (g & 1)] = d;   // keys 16 (kb & 1) + 4 g + i of the half
+                    d[0] = pack_f16_rne(P[0], P[1]);
+                    d[1] = pack_f16_rne(P[2], P[3]);
+                    *(u32x2 *)&X.p[hh][kb >> 1][2 * (kb & 1) + (g >> 1)][n][2 * (g & 1)] = d;   // keys 16 (kb & 1) + 4 g + i of the half
                 }
                 if (g == 0) X.m[hh][n][kb] = m_loc;
-                if (lane == 0) X.e[hh][kb] = e_loc;
             }
-            valid_nxt = valid_aft;
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of tile t+2 has landed
             LDS_BARRIER();
         }
 
@@ -431,58 +408,100 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         for (int h2 = 0; h2 < 2; h2++)
 #pragma unroll
             for (int j = 0; j < 8; j++) oacc[h2][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        int e_run = E_NONE;                               // 2^e_run is above every scale of this wave's block seen so far
+        // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; in the loop only the value
+        // waves copy (the scoring waves are the long pole of a step, and a wave that issues copies
+        // stalls while the memory pipeline takes them): wave cw takes pieces cw, cw + 4, ...
+        auto issue_value = [&](int r, Tile *b) {
+            const int64_t rc = r >= 0 ? r : 0;            // masked positions fetch row 0, weight 0
+#pragma unroll
+            for (int i = 0; i < 11; i++) {
+                const int pc = cw + 4 * i;
+                if (pc < NCOL) dma16(rows + rc * KDIM + 16 * pc, &b->kv[pc][0][0]);
+                else if (pc < NCOL + NBLK) dma4(scales + rc * NBLK + (pc - NCOL), &b->sc[pc - NCOL][0]);
+            }
+        };
         asm volatile("" ::: "memory");
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
-            if (t >= 0 && t + 2 < n_tiles) {
-                const int r2 = row_of(t + 2);
-                issue(r2, &sm.tile[(t + 2) % NST]);       // the stage tile t-1 left at the last barrier
-                valid_aft = __ballot(r2 >= 0);
-            }
+            const bool do_copy = t >= 0 && t + 3 < n_tiles;
+            if (do_copy) issue_value(row_of(t + 3), &sm.tile[(t + 3) % NST]);   // the stage tile t-1 left at the last barrier
             if (t >= 0) {
-                // ---- values O^T[dim][head] += V^T P^T for dims 128 cw.., all 32 heads, tile t ----
+                // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 32 heads, tile t ----
                 const Tile &T = sm.tile[t % NST];
                 const Xch &X = sm.x[t & 1];
                 const uint8_t *vbase = &T.kv[0][0][0] + tr_off;
+                // scales of this wave's block for the keys of this lane's contraction slots
+                f32x4 sv[2][2];
+#pragma unroll
+                for (int kh = 0; kh < 2; kh++)
+#pragma unroll
+                    for (int q = 0; q < 2; q++) sv[kh][q] = *(const f32x4 *)&T.sc[vblk][32 * kh + 8 * g + 4 * q];
                 u32x4 pw[2][2];                           // [head half][key half]
                 f32x4 ml[2];
 #pragma unroll
                 for (int h2 = 0; h2 < 2; h2++) {
 #pragma unroll
-                    for (int kh = 0; kh < 2; kh++) pw[h2][kh] = *(const u32x4 *)&X.w[vblk][h2][kh][g][n][0];
+                    for (int kh = 0; kh < 2; kh++) pw[h2][kh] = *(const u32x4 *)&X.p[h2][kh][g][n][0];
                     ml[h2] = *(const f32x4 *)&X.m[h2][n][0];
                 }
-                // the exponents the key blocks used (the two head halves agree: same keys, same rule)
-                const i32x4 el = *(const i32x4 *)&X.e[0][0];
-                const int e01 = el[0] > el[1] ? el[0] : el[1], e23 = el[2] > el[3] ? el[2] : el[3];
-                const int e_t = e01 > e23 ? e01 : e23;
-                const int e_new = e_t > e_ref ? e_t : e_ref;
-                const bool e_moved = e_new != e_ref || el[0] != e_new || el[1] != e_new || el[2] != e_new || el[3] != e_new;
+                // normaliser of the fp16 weights: a power of two above every scale seen so far (it
+                // only grows, and only then the lanes confer)
+                float ecorr = 1.0f;
+                {
+                    float smax = fmaxf(fmaxf(fmaxf(sv[0][0][0], sv[0][0][1]), fmaxf(sv[0][0][2], sv[0][0][3])),
+                                       fmaxf(fmaxf(sv[0][1][0], sv[0][1][1]), fmaxf(sv[0][1][2], sv[0][1][3])));
+                    smax = fmaxf(smax, fmaxf(fmaxf(fmaxf(sv[1][0][0], sv[1][0][1]), fmaxf(sv[1][0][2], sv[1][0][3])),
+                                             fmaxf(fmaxf(sv[1][1][0], sv[1][1][1]), fmaxf(sv[1][1][2], sv[1][1][3]))));
+                    const float thr = e_run == E_NONE ? 0.0f : pow2i(e_run);   // scales below 2^e_run fit
+                    if (__any(smax >= thr && smax > 0.0f)) {
+#pragma unroll
+                        for (int o = 32; o > 0; o >>= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
+                        const int e_tile = (int)((__builtin_bit_cast(uint32_t, smax) >> 23) & 0xFFu) - 126;
+                        if (e_tile > e_run) {
+                            if (e_run != E_NONE) ecorr = pow2i(e_run - e_tile);
+                            e_run = e_tile;
+                        }
+                    }
+                }
+                const float wfac = e_run == E_NONE ? 0.0f : pow2i(WEXP - e_run);
+                u32x4 sw[2];                              // scale * 2^(WEXP - e_run) of the slots' keys, fp16 pairs
+#pragma unroll
+                for (int kh = 0; kh < 2; kh++) {
+                    sw[kh][0] = pack_f16_rne(sv[kh][0][0] * wfac, sv[kh][0][1] * wfac);
+                    sw[kh][1] = pack_f16_rne(sv[kh][0][2] * wfac, sv[kh][0][3] * wfac);
+                    sw[kh][2] = pack_f16_rne(sv[kh][1][0] * wfac, sv[kh][1][1] * wfac);
+                    sw[kh][3] = pack_f16_rne(sv[kh][1][2] * wfac, sv[kh][1][3] * wfac);
+                }
 #pragma unroll
                 for (int h2 = 0; h2 < 2; h2++) {
                     const float m_new = fmaxf(m_ref[h2], fmaxf(fmaxf(ml[h2][0], ml[h2][1]), fmaxf(ml[h2][2], ml[h2][3])));
-                    if (e_moved || __any(m_new != m_ref[h2] || ml[h2][0] != m_new || ml[h2][1] != m_new || ml[h2][2] != m_new || ml[h2][3] != m_new)) {
+                    float fsel0 = 1.0f, fsel1 = 1.0f;
+                    const bool moved = __any(m_new != m_ref[h2] || ml[h2][0] != m_new || ml[h2][1] != m_new || ml[h2][2] != m_new || ml[h2][3] != m_new);
+                    if (moved || ecorr != 1.0f) {
                         float f[4];
 #pragma unroll
-                        for (int k = 0; k < 4; k++)
-                            f[k] = (ml[h2][k] == -INFINITY || el[k] == E_NONE) ? 0.0f : __builtin_amdgcn_exp2f(ml[h2][k] - m_new) * pow2i(el[k] - e_new);
-                        const float c = (m_ref[h2] == -INFINITY || e_ref == E_NONE) ? 1.0f : __builtin_amdgcn_exp2f(m_ref[h2] - m_new) * pow2i(e_ref - e_new);
+                        for (int k = 0; k < 4; k++) f[k] = ml[h2][k] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[h2][k] - m_new);
+                        const float c = (m_ref[h2] == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref[h2] - m_new)) * ecorr;
                         m_ref[h2] = m_new;
 #pragma unroll
                         for (int j = 0; j < 8; j++) oacc[h2][j] *= c;
-                        // weights were taken relative to each key block's own reference: bring them to m_new
-                        // (slot group g of half kh holds keys of key block 2 kh + g / 2)
-                        const float fsel0 = (g >> 1) ? f[1] : f[0], fsel1 = (g >> 1) ? f[3] : f[2];
+                        // probabilities were taken relative to each key block's own reference: bring
+                        // them to m_new (slot group g of half kh holds keys of key block 2 kh + g / 2)
+                        fsel0 = (g >> 1) ? f[1] : f[0];
+                        fsel1 = (g >> 1) ? f[3] : f[2];
+                    }
 #pragma unroll
-                        for (int kh = 0; kh < 2; kh++)
+                    for (int kh = 0; kh < 2; kh++) {
+                        u32x4 swf = sw[kh];
+                        if (moved) {
 #pragma unroll
-                            for (int d = 0; d < 4; d++) {
-                                const float fk = kh ? fsel1 : fsel0;
-                                pw[h2][kh][d] = scale_f16x2(pw[h2][kh][d], fk);
-                            }
+                            for (int d = 0; d < 4; d++) swf[d] = scale_f16x2(swf[d], kh ? fsel1 : fsel0);
+                        }
+#pragma unroll
+                        for (int d = 0; d < 4; d++) pw[h2][kh][d] = mul_f16x2(pw[h2][kh][d], swf[d]);
                     }
                 }
-                e_ref = e_new;
 #pragma unroll
                 for (int j0 = 0; j0 < 8; j0 += 4) {
                     i32x2 vt[4][2];
@@ -506,8 +525,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                         }
                 }
             }
-            valid_nxt = valid_aft;
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of tile t+2 has landed
+            // tile t+2 must be whole at the next barrier; the copies of tile t+3, issued in this
+            // step (eleven by value wave 0, ten by the others), may stay in flight
+            if (!do_copy) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else if (cw == 0) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
             LDS_BARRIER();
         }
 
@@ -520,7 +542,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             const float L = (lv[0] + lv[1]) + (lv[2] + lv[3]);
             const int head = hb * HW + 16 * h2 + n;
             if (head >= p.nh) continue;
-            const float unit_f = e_ref == E_NONE ? 0.0f : pow2i(e_ref - WEXP);   // the accumulators are in units of 2^(e_ref - WEXP)
+            const float unit_f = e_run == E_NONE ? 0.0f : pow2i(e_run - WEXP);   // the accumulators are in units of 2^(e_run - WEXP)
             const float fin = p.n_splits == 1 ? (L > 0.0f ? unit_f / L : 0.0f) : unit_f;
             const size_t pb = ((size_t)y * p.n_splits + split) * (2 * n_hb) + 2 * hb + h2;
 #pragma unroll
