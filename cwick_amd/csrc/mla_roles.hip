@@ -25,11 +25,12 @@
 //   one step later -- almost always a comparison and nothing else.  Each scoring lane keeps the
 //   sum of its own keys; the sums meet once, after the loop.
 //   Tiles are copied global -> LDS by global_load_lds (no registers) into four stages: tile t+3
-//   is fetched during step t, two tiles ahead of its first use.  In the loop only the value
-//   waves issue copies: a wave that issues them stalls while the memory pipeline takes them, and
-//   the scoring waves are the long pole of a step.  The copies are issued from inline assembly
-//   and the barrier waits for LDS traffic only, so the compiler never makes anything wait for
-//   the tiles in flight.
+//   is fetched during step t, two tiles ahead of its first use.  A wave that issues copies stalls
+//   while the memory pipeline takes them, so they go where there is slack: the value waves issue
+//   three each at the top of the step, the scoring waves the rest at the end of theirs, when they
+//   would otherwise wait at the barrier.  The copies are issued from inline assembly and the
+//   barrier waits for LDS traffic only, so the compiler never makes anything wait for the tiles
+//   in flight.
 //
 //   LDS tile layout [16-byte column][key 0..63][16 B]: the K fragment is two 16-byte reads per
 //   lane, 256 B contiguous per 16 keys; the V^T fragment of 32 keys x 16 dims is one
@@ -73,6 +74,7 @@ constexpr int TK = 64;                        // keys per tile
 constexpr int HB = 16;                        // heads per head half (partials are laid out per 16 heads)
 constexpr int HW = 32;                        // heads per workgroup
 constexpr int NST = 4;                        // tile stages
+constexpr int NV = 3;                         // copies per tile a value wave issues (the scoring waves take the rest)
 constexpr int NCOL = KDIM / 16;               // 36 sixteen-byte columns per row
 constexpr int NDB = VDIM / 16;                // 32 sixteen-dim output blocks
 constexpr float LAZY = 4.0f;                  // the reference moves when a tile exceeds it by 2^LAZY
@@ -206,6 +208,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         if (wave < 5) dma4(scales + rc * NBLK + wave, &b->sc[wave][0]);
     };
 
+    // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks
+    auto piece = [&](int pc, int64_t rc, Tile *b) {
+        if (pc < NCOL) dma16(rows + rc * KDIM + 16 * pc, &b->kv[pc][0][0]);
+        else if (pc < NCOL + NBLK) dma4(scales + rc * NBLK + (pc - NCOL), &b->sc[pc - NCOL][0]);
+    };
     {
         const int row0 = row_of(0), row1 = row_of(1), row2 = row_of(2);
         if (n_tiles > 0) issue(row0, &sm.tile[0]);
@@ -309,6 +316,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         for (int t = -1; t < n_tiles; t++) {
             const int row_now = row_nxt;              // rows of tile t+1, fetched one step ahead
             row_nxt = row_of(t + 2);
+            const bool do_copy = t >= 0 && t + 3 < n_tiles;
+            const int row_cp = do_copy ? row_of(t + 3) : 0;
             if (t >= 0) {
                 // what the four key blocks of tile t used as reference for this half's heads
                 const f32x4 ml = *(const f32x4 *)&sm.x[t & 1].m[hh][n][0];
@@ -392,6 +401,14 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 }
                 if (g == 0) X.m[hh][n][kb] = m_loc;
             }
+            // the copies this wave issued a step ago (its share of tile t+2) have long landed; its
+            // share of tile t+3 goes out now, when the wave would otherwise wait at the barrier
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (do_copy) {
+                const int64_t rc = row_cp >= 0 ? row_cp : 0;
+#pragma unroll
+                for (int i = 0; i < (NCOL + NBLK - 4 * NV + 7) / 8; i++) piece(4 * NV + wave + 8 * i, rc, &sm.tile[(t + 3) % NST]);
+            }
             LDS_BARRIER();
         }
 
@@ -415,11 +432,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         auto issue_value = [&](int r, Tile *b) {
             const int64_t rc = r >= 0 ? r : 0;            // masked positions fetch row 0, weight 0
 #pragma unroll
-            for (int i = 0; i < 11; i++) {
-                const int pc = cw + 4 * i;
-                if (pc < NCOL) dma16(rows + rc * KDIM + 16 * pc, &b->kv[pc][0][0]);
-                else if (pc < NCOL + NBLK) dma4(scales + rc * NBLK + (pc - NCOL), &b->sc[pc - NCOL][0]);
-            }
+            for (int i = 0; i < NV; i++) piece(cw + 4 * i, rc, b);
         };
         asm volatile("" ::: "memory");
 #pragma clang loop unroll(disable)
@@ -528,8 +541,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             // tile t+2 must be whole at the next barrier; the copies of tile t+3, issued in this
             // step (eleven by value wave 0, ten by the others), may stay in flight
             if (!do_copy) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            else if (cw == 0) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NV) : "memory");
             LDS_BARRIER();
         }
 
