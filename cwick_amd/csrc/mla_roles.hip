@@ -426,6 +426,9 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 #pragma unroll
             for (int j = 0; j < 8; j++) oacc[h2][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
         int e_run = E_NONE;                               // 2^e_run is above every scale of this wave's block seen so far
+        // the value wave shares its SIMD with two scoring waves that stream MFMAs: without priority
+        // its many short VALU instructions wait behind them and it becomes the long pole of the step
+        __builtin_amdgcn_s_setprio(3);
         // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; in the loop only the value
         // waves copy (the scoring waves are the long pole of a step, and a wave that issues copies
         // stalls while the memory pipeline takes them): wave cw takes pieces cw, cw + 4, ...
