@@ -213,12 +213,10 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         if (pc < NCOL) dma16(rows + rc * KDIM + 16 * pc, &b->kv[pc][0][0]);
         else if (pc < NCOL + NBLK) dma4(scales + rc * NBLK + (pc - NCOL), &b->sc[pc - NCOL][0]);
     };
-    {
-        const int row0 = row_of(0), row1 = row_of(1), row2 = row_of(2);
-        if (n_tiles > 0) issue(row0, &sm.tile[0]);
-        if (n_tiles > 1) issue(row1, &sm.tile[1]);
-        if (n_tiles > 2) issue(row2, &sm.tile[2]);
-    }
+    // Only tile 0 is fetched before the loop, by everybody.  In step -1, while tile 0 is scored,
+    // the value waves (nothing to accumulate yet) fetch tile 1, and the scoring waves fetch tile 2
+    // at the end of their step; from step 0 on tile t+3 is fetched during step t.
+    if (n_tiles > 0) issue(row_of(0), &sm.tile[0]);
 
     // ---- Q for 2 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
     // 128-dim block (the hardware pairs the scale of lane (n, g) with k-elements that live in other
@@ -274,7 +272,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             }
             qp->sc[lane] = 127 + s;
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tiles 0, 1 and 2 have landed (this wave's share)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tile 0 has landed (this wave's share)
         LDS_BARRIER();
     }
 
@@ -316,7 +314,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         for (int t = -1; t < n_tiles; t++) {
             const int row_now = row_nxt;              // rows of tile t+1, fetched one step ahead
             row_nxt = row_of(t + 2);
-            const bool do_copy = t >= 0 && t + 3 < n_tiles;
+            const bool do_copy = t + 3 < n_tiles;
             const int row_cp = do_copy ? row_of(t + 3) : 0;
             if (t >= 0) {
                 // what the four key blocks of tile t used as reference for this half's heads
@@ -406,8 +404,13 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (do_copy) {
                 const int64_t rc = row_cp >= 0 ? row_cp : 0;
+                if (t >= 0) {
 #pragma unroll
-                for (int i = 0; i < (NCOL + NBLK - 4 * NV + 7) / 8; i++) piece(4 * NV + wave + 8 * i, rc, &sm.tile[(t + 3) % NST]);
+                    for (int i = 0; i < (NCOL + NBLK - 4 * NV + 7) / 8; i++) piece(4 * NV + wave + 8 * i, rc, &sm.tile[(t + 3) % NST]);
+                } else {                              // all of tile 2
+#pragma unroll
+                    for (int i = 0; i < (NCOL + NBLK + 7) / 8; i++) piece(wave + 8 * i, rc, &sm.tile[2]);
+                }
             }
             LDS_BARRIER();
         }
@@ -442,6 +445,12 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         for (int t = -1; t < n_tiles; t++) {
             const bool do_copy = t >= 0 && t + 3 < n_tiles;
             if (do_copy) issue_value(row_of(t + 3), &sm.tile[(t + 3) % NST]);   // the stage tile t-1 left at the last barrier
+            if (t < 0 && n_tiles > 1) {                   // all of tile 1
+                const int r = row_of(1);
+                const int64_t rc = r >= 0 ? r : 0;
+#pragma unroll
+                for (int i = 0; i < (NCOL + NBLK + 3) / 4; i++) piece(cw + 4 * i, rc, &sm.tile[1]);
+            }
             if (t >= 0) {
                 // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 32 heads, tile t ----
                 const Tile &T = sm.tile[t % NST];
