@@ -12,24 +12,36 @@
 //   query heads of the kv head times P = 256/GROUP consecutive positions
 //   (heads-as-M: K and V tiles are read once for all heads of the group).
 //   Key tiles of TK = 32.  K and V go global -> LDS by global_load_lds_dwordx4
-//   (no staging registers), two tiles ahead for K and one for V, one workgroup
-//   barrier per tile.
+//   (no staging registers), one workgroup barrier per tile.
 //   scores:  S^T[key][row] = K[key][dim] . Q^T[dim][row], v_mfma_f32_32x32x16_bf16,
-//            K fragments from LDS, Q fragments resident in registers (80 of 128; the rest re-read from LDS).
+//            K fragments from LDS, Q fragments of the first column block resident in
+//            registers, those of the second re-read from a per-lane LDS park.
 //            One query row per lane column: softmax statistics are per-lane.
+//            The score accumulators are pinned to VGPRs (inline assembly): through the
+//            builtin every MFMA result is placed in AGPRs, which the outputs fill.
 //   values:  O^T[dim][row] += V^T[dim][key] . P^T[key][row].  P^T is the score
 //            accumulator itself (rounded to bf16) -- its register layout is the
 //            B-operand layout once the contraction slots are numbered to match;
 //            V^T fragments come out of the V tile through the LDS transpose read
 //            (ds_read_b64_tr_b16).  The 256 output registers live in AGPRs.
-//   schedule: one wave per SIMD, so the loop is software-pipelined by hand: the
-//            body computes the scores of tile t+1, and then the softmax of tile
-//            t+1 (VALU) next to the value MFMAs of tile t.
+//   schedule: one wave per SIMD, so the loop is software-pipelined by hand, three
+//            tiles deep: step t interleaves, MFMA by MFMA, the scores of tile t+2, the
+//            softmax of tile t+1 (VALU, in the shadow of the matrix instructions) and
+//            the value products of tile t.  The barrier that opens step t+1 sits near
+//            the end of step t and the first fragments of step t+1 are fetched behind
+//            it, so the matrix pipe does not drain between steps.  K is copied three
+//            tiles ahead into two buffers, V two tiles ahead into three: a tile costs
+//            about 1400 cycles of the CU's copy path, so the copies are spread over the
+//            whole step and only K has to land within it.
 //   The softmax reference of a row is the maximum of its first tile and stays
 //   there while later scores exceed it by less than 64 (log2 units): weights up
 //   to 2^64 lose nothing in bf16 or fp32.  A wave that meets a larger score
 //   leaves the fast loop for a slow one that moves the reference and rescales
 //   the accumulators (in place, in AGPRs) every tile.
+//   Position blocks that see at most 2048 keys run the PRECISE variant (the
+//   rounding residual of the weights goes through the matrix core too) in the
+//   simpler two-stage schedule: scores of tile t+1, then its softmax next to
+//   the value products of tile t.
 //
 //   LDS tile layout: 16 blocks of 1 KiB (+64 B pad), block b = 16-byte columns
 //   2b and 2b+1 of all 32 keys, slot (c&1)*32 + (key ^ 8(c&1)).  A K fragment
@@ -54,9 +66,9 @@ typedef __attribute__((address_space(3))) void pf_lds_void;
 
 struct PfSmem {
     unsigned char k[2][PF_TILE];
-    unsigned char v[2][PF_TILE];
+    unsigned char v[3][PF_TILE];                // the pipelined body keeps three V tiles, the other two
     // Q fragments of column block B, k-steps PF_QX0..15, parked per lane: the register file
-    // holds 256 accumulators + 80 Q registers + the working set, not 128 Q registers
+    // holds 256 accumulators + 64 Q registers + the working set, not 128 Q registers
     u32x4 qx[PF_THREADS / 64][16 - PF_QX0][64];
 };
 
@@ -168,9 +180,19 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     // scores of one tile for both column blocks
     // One wave per SIMD: nothing hides an LDS round trip, so the fragments are fetched PF_PRE
     // k-steps ahead of the MFMAs that use them.
-    // copy_t >= 0: the copies of K(copy_t + 2) and V(copy_t + 1) are issued between the MFMAs
-    // (an LDS-DMA instruction occupies the issue slot for about as long as two MFMAs run)
-    auto scores = [&](int tile, f32x16 (&s)[2], int copy_t) {
+    // Score MFMA with its accumulator pinned to VGPRs: through the builtin the allocator places
+    // every MFMA result in AGPRs, which the 256 output accumulators fill, and moves registers
+    // back and forth every tile.  Opaque to the compiler's hazard tracking: score_done() goes
+    // between the last MFMA and the first VALU read of the result.
+    auto score_mfma = [&](f32x16 &acc, bf16x8 a, bf16x8 b, bool first) {
+        if (first) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    };
+    auto score_done = [&]() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); };
+    // ck / cv >= 0: the copies of K(ck) and V(cv) are issued between the MFMAs (an LDS-DMA
+    // instruction occupies the issue slot for about as long as two MFMAs run).  Tile u of K or V
+    // lives in buffer u & 1.
+    auto scores = [&](int tile, f32x16 (&s)[2], int ck, int cv) {
         const unsigned char *kb = &sm.k[tile & 1][0] + kfrag_off;
         const u32x4 *qb = &sm.qx[wave][0][lane];
         u32x4 ka[PF_PRE], qa[PF_PRE];
@@ -179,15 +201,11 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
             ka[ks] = *(const u32x4 *)(kb + ks * PF_BLK);
             if (ks >= PF_QX0) qa[ks] = qb[(ks - PF_QX0) * 64];
         }
-        const bool do_k = copy_t >= 0 && copy_t + 2 < n_tiles, do_v = copy_t >= 0;
-        const uint16_t *src_k = copy_src(Kg, do_k ? copy_t + 2 : 0);
-        const uint16_t *src_v = copy_src(Vg, do_v ? copy_t + 1 : 0);
-        const uint32_t dst_k = lds_k + (uint32_t)((copy_t & 1) * PF_TILE);
-        const uint32_t dst_v = lds_v + (uint32_t)(((copy_t + 1) & 1) * PF_TILE);
-#pragma unroll
-        for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[c][i] = 0.0f;
+        const bool do_k = ck >= 0 && ck < n_tiles, do_v = cv >= 0 && cv < n_tiles;
+        const uint16_t *src_k = copy_src(Kg, do_k ? ck : 0);
+        const uint16_t *src_v = copy_src(Vg, do_v ? cv : 0);
+        const uint32_t dst_k = lds_k + (uint32_t)((ck & 1) * PF_TILE);
+        const uint32_t dst_v = lds_v + (uint32_t)((cv & 1) * PF_TILE);
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
             const bf16x8 kf = __builtin_bit_cast(bf16x8, ka[ks % PF_PRE]);
@@ -196,13 +214,30 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                 ka[ks % PF_PRE] = *(const u32x4 *)(kb + (ks + PF_PRE) * PF_BLK);
                 if (ks + PF_PRE >= PF_QX0) qa[ks % PF_PRE] = qb[(ks + PF_PRE - PF_QX0) * 64];
             }
-            s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
-            s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q1, s[1], 0, 0, 0);
+            score_mfma(s[0], kf, qf[0][ks], ks == 0);
+            score_mfma(s[1], kf, q1, ks == 0);
             if ((ks & 1) == 0) {
                 if (ks < 8) { if (do_k) copy_one(src_k, dst_k, ks >> 1); }
                 else if (do_v) copy_one(src_v, dst_v, (ks - 8) >> 1);
             }
         }
+        score_done();
+    };
+    // the same from global memory (the slow loop of the pipelined body: its K tile has already
+    // been overwritten in LDS)
+    auto scores_global = [&](int tile, f32x16 (&s)[2]) {
+        int64_t row = (int64_t)tile * PF_TK + l32;
+        if (row > n_keys_all - 1) row = n_keys_all - 1;             // masked anyway
+        const uint16_t *kr = K + row * kv_stride + (size_t)kvh * PF_HD + 8 * g;
+        const u32x4 *qb = &sm.qx[wave][0][lane];
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            const bf16x8 kf = __builtin_bit_cast(bf16x8, *(const u32x4 *)(kr + 16 * ks));
+            const bf16x8 q1 = ks < PF_QX0 ? qf[1][ks] : __builtin_bit_cast(bf16x8, qb[(ks - PF_QX0) * 64]);
+            score_mfma(s[0], kf, qf[0][ks], ks == 0);
+            score_mfma(s[1], kf, q1, ks == 0);
+        }
+        score_done();
     };
     // softmax bookkeeping of one tile and column block, in two parts.
     // register i holds key (i/4)*8 + 4g + i%4 of the tile for this lane's row.
@@ -229,11 +264,13 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             s[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale_log2e, -m_use));   // masked: 0
-            psum += s[i];
+            if (precise) psum += s[i];
         }
-        l_part[c] += psum;
         // contraction slot (g, jj) of step ks2 <-> tile key 16*ks2 + (jj/4)*8 + 4g + jj%4,
         // i.e. score register 8*ks2 + jj: P^T needs no data movement.
+        // With single-term weights the row sum is the sum of the ROUNDED weights: the output is
+        // then a convex combination of value rows whatever the rounding did (a row dominated by
+        // one key is exact), and the error is 2^-9 of the spread of the values, not of their size.
 #pragma unroll
         for (int ks2 = 0; ks2 < 2; ks2++)
 #pragma unroll
@@ -242,7 +279,10 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                 if (precise)
                     pl[ks2][h] = pack_bf16_rne(s[8 * ks2 + 2 * h] - bf16lo_to_f32(pw[ks2][h]),
                                                s[8 * ks2 + 2 * h + 1] - bf16hi_to_f32(pw[ks2][h]));
+                else
+                    psum += bf16lo_to_f32(pw[ks2][h]) + bf16hi_to_f32(pw[ks2][h]);
             }
+        l_part[c] += psum;
     };
     // The running reference m_ref is the row maximum of tile 0 and stays there while later tiles
     // exceed it by less than 2^SLACK: weights up to 2^SLACK are as exact in bf16 and fp32 as
@@ -260,7 +300,7 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     };
     // value MFMAs of one tile for both column blocks
     auto values = [&](int tile, const u32x4 (&pw)[2][2], const u32x4 (&pl)[2][2]) {
-        const unsigned char *vb = &sm.v[tile & 1][0];
+        const unsigned char *vb = &sm.v[PRECISE ? (tile & 1) : (tile % 3)][0];
         // step st = 8 ks2 + db; its two transpose reads are issued PF_PRE steps ahead
         s16x4 lo[PF_PRE], hi[PF_PRE];
         auto fetch = [&](int st, int slot) {
@@ -301,77 +341,52 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                                  : "v"(corr[c]));
                 }
     };
-    // top of step t: K(t+1) and V(t) have landed (this wave's part, then everyone's; all reads of
-    // step t-1 are over as well, so the copies of K(t+2) and V(t+1) may start)
+    // top of step t: the tiles step t reads have landed (this wave's part, then everyone's), and
+    // all reads of step t-1 are over, so the copies of step t may overwrite its buffers
     auto step_top = [&]() {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         PF_LDS_BARRIER();
     };
 
-    // ---- prologue: K(0), V(0), K(1); scores and softmax of tile 0 (sets the reference) ----
-    issue(Kg, lds_k, 0);
-    issue(Vg, lds_v, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    PF_LDS_BARRIER();
-    if (n_tiles > 1) issue(Kg, lds_k + PF_TILE, 1);
+    if constexpr (PRECISE) {
+        // ---- prologue: K(0), V(0), K(1); scores and softmax of tile 0 (sets the reference) ----
+        issue(Kg, lds_k, 0);
+        issue(Vg, lds_v, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PF_LDS_BARRIER();
+        if (n_tiles > 1) issue(Kg, lds_k + PF_TILE, 1);
 
-    u32x4 pw[2][2], pl[2][2];
-    {
-        f32x16 s[2];
-        scores(0, s, -1);
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            (void)sm_move_ref(c, sm_prep(0, c, s[c]));                  // nothing accumulated yet
-            sm_finish(c, s[c], pw[c], pl[c]);
-        }
-    }
-
-    // ---- fast loop: scores(t+1); then softmax(t+1) beside values(t); no rescale.  The softmax
-    // is speculative: whether a row outgrew the reference is looked at after the MFMAs.
-    int t = 0;
-    bool slow = false;
-    for (; t + 1 < n_tiles; t++) {
-        step_top();
-        f32x16 s[2];
-        scores(t + 1, s, t);
-        u32x4 pwn[2][2], pln[2][2];
-        const float l_save[2] = {l_part[0], l_part[1]};
-        const float x0 = sm_prep(t + 1, 0, s[0]), x1 = sm_prep(t + 1, 1, s[1]);
-        sm_finish(0, s[0], pwn[0], pln[0]);
-        sm_finish(1, s[1], pwn[1], pln[1]);
-        values(t, pw, pl);
-        if (__any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK)) {   // a row outgrew the reference
-            l_part[0] = l_save[0];
-            l_part[1] = l_save[1];
-            slow = true;
-            break;
-        }
-#pragma unroll
-        for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int k2 = 0; k2 < 2; k2++) {
-                pw[c][k2] = pwn[c][k2];
-                pl[c][k2] = pln[c][k2];
-            }
-    }
-    // ---- slow loop (rare): the reference follows the maximum, accumulators rescaled every tile.
-    // It resumes step t after its top, copies and values(t); the scores are recomputed.
-    if (slow) {
-        bool resumed = true;
-        for (; t + 1 < n_tiles; t++) {
-            if (!resumed) step_top();
+        u32x4 pw[2][2], pl[2][2];
+        {
             f32x16 s[2];
-            scores(t + 1, s, resumed ? -1 : t);
-            u32x4 pwn[2][2], pln[2][2];
-            float corr[2];
+            scores(0, s, -1, -1);
 #pragma unroll
             for (int c = 0; c < 2; c++) {
-                corr[c] = sm_move_ref(c, sm_prep(t + 1, c, s[c]));
-                sm_finish(c, s[c], pwn[c], pln[c]);
+                (void)sm_move_ref(c, sm_prep(0, c, s[c]));                  // nothing accumulated yet
+                sm_finish(c, s[c], pw[c], pl[c]);
             }
-            if (!resumed) values(t, pw, pl);
-            resumed = false;
-            rescale(corr);
+        }
+
+        // ---- fast loop: scores(t+1); then softmax(t+1) beside values(t); no rescale.  The softmax
+        // is speculative: whether a row outgrew the reference is looked at after the MFMAs.
+        int t = 0;
+        bool slow = false;
+        for (; t + 1 < n_tiles; t++) {
+            step_top();
+            f32x16 s[2];
+            scores(t + 1, s, t + 2, t + 1);
+            u32x4 pwn[2][2], pln[2][2];
+            const float l_save[2] = {l_part[0], l_part[1]};
+            const float x0 = sm_prep(t + 1, 0, s[0]), x1 = sm_prep(t + 1, 1, s[1]);
+            sm_finish(0, s[0], pwn[0], pln[0]);
+            sm_finish(1, s[1], pwn[1], pln[1]);
+            values(t, pw, pl);
+            if (__any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK)) {   // a row outgrew the reference
+                l_part[0] = l_save[0];
+                l_part[1] = l_save[1];
+                slow = true;
+                break;
+            }
 #pragma unroll
             for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -380,11 +395,236 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                     pl[c][k2] = pln[c][k2];
                 }
         }
+        // ---- slow loop (rare): the reference follows the maximum, accumulators rescaled every tile.
+        // It resumes step t after its top, copies and values(t); the scores are recomputed.
+        if (slow) {
+            bool resumed = true;
+            for (; t + 1 < n_tiles; t++) {
+                if (!resumed) step_top();
+                f32x16 s[2];
+                scores(t + 1, s, resumed ? -1 : t + 2, resumed ? -1 : t + 1);
+                u32x4 pwn[2][2], pln[2][2];
+                float corr[2];
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    corr[c] = sm_move_ref(c, sm_prep(t + 1, c, s[c]));
+                    sm_finish(c, s[c], pwn[c], pln[c]);
+                }
+                if (!resumed) values(t, pw, pl);
+                resumed = false;
+                rescale(corr);
+#pragma unroll
+                for (int c = 0; c < 2; c++)
+#pragma unroll
+                    for (int k2 = 0; k2 < 2; k2++) {
+                        pw[c][k2] = pwn[c][k2];
+                        pl[c][k2] = pln[c][k2];
+                    }
+            }
+        }
+        // ---- last tile's values ----
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PF_LDS_BARRIER();
+        values(n_tiles - 1, pw, pl);
+
+    } else {
+        // ---- pipelined body: step t computes the scores of tile t+2, the softmax of tile t+1 and the
+        // value products of tile t, interleaved MFMA by MFMA so that the softmax (VALU), the fragment
+        // reads (LDS) and the copies issue in the shadow of the matrix instructions.  The loop is
+        // rotated: the barrier that opens step t+1 sits in slot 14 of step t (by then every
+        // fragment read of step t has returned and the copies issued in slots 0..7 have landed), and
+        // slots 14 and 15 already fetch the first fragments of step t+1, so the matrix pipe does not
+        // drain between steps.  Only tiles below the diagonal take this form; the (at most three)
+        // tiles on it and the tail run in sequence.
+        constexpr float BIG = 18446744073709551616.0f;                  // 2^SLACK
+        u32x4 ka[2], qa[2];                                             // fragments of the next two slots
+        s16x4 lo[2], hi[2];
+        auto fetch = [&](int t, int i, int slot) {                      // fragments of slot i of step t
+            const unsigned char *kb = &sm.k[t & 1][0] + kfrag_off;      // K(t+2)
+            const unsigned char *vb = &sm.v[t % 3][0];                  // V(t)
+            ka[slot] = *(const u32x4 *)(kb + i * PF_BLK);
+            if (i >= PF_QX0) qa[slot] = sm.qx[wave][i - PF_QX0][lane];
+            const int ks2 = i >> 3, db = i & 7;
+            lo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][0] + db * (2 * PF_BLK)));
+            hi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + v_off[ks2][1] + db * (2 * PF_BLK)));
+        };
+        // the running sums as opaque instructions: left to the compiler, the thirty-two additions
+        // of a step sink to its end, a dependent chain behind the last MFMA
+        auto psum_add = [&](float &acc, float x) { asm volatile("v_add_f32 %0, %1, %0" : "+v"(acc) : "v"(x)); };
+        auto pstep = [&](int t, f32x16 (&sc)[2], f32x16 (&sn)[2], const u32x4 (&pc)[2][2],
+                         u32x4 (&pn)[2][2], float (&ps)[2]) {
+            const uint16_t *src_k = copy_src(Kg, t + 3);     // past the last tile: clipped rows into a dead buffer
+            const uint16_t *src_v = copy_src(Vg, t + 2);
+            const uint32_t dst_k = lds_k + (uint32_t)(((t + 1) & 1) * PF_TILE);
+            const uint32_t dst_v = lds_v + (uint32_t)(((t + 2) % 3) * PF_TILE);
+            const float mu0 = m_ref[0], mu1 = m_ref[1];
+            float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                typedef __attribute__((ext_vector_type(8))) short s16x8;
+                const int ks2 = i >> 3, db = i & 7;
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, ka[i & 1]);
+                const bf16x8 q1 = i < PF_QX0 ? qf[1][i] : __builtin_bit_cast(bf16x8, qa[i & 1]);
+                const bf16x8 va = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo[i & 1], hi[i & 1], 0, 1, 2, 3, 4, 5, 6, 7));
+                score_mfma(sn[0], kf, qf[0][i], i == 0);
+                sc[0][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][i], scale_log2e, -mu0));
+                __builtin_amdgcn_sched_barrier(0);
+                oacc[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pc[0][ks2]), oacc[0][db], 0, 0, 0);
+                sc[1][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[1][i], scale_log2e, -mu1));
+                __builtin_amdgcn_sched_barrier(0);
+                score_mfma(sn[1], kf, q1, i == 0);
+                if (i == 14) {                                       // the top of step t+1
+                    // all but this step's three V copies: K(t+3) and V(t+1) have landed
+                    asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+                    PF_LDS_BARRIER();
+                }
+                if (i < 14) fetch(t, i + 2, i & 1);
+                else fetch(t + 1, i - 14, i & 1);
+                __builtin_amdgcn_sched_barrier(0);
+                oacc[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pc[1][ks2]), oacc[1][db], 0, 0, 0);
+                if (i & 1) {                                         // weights, and the sum of the rounded weights
+                    const uint32_t w0 = pack_bf16_rne(sc[0][i - 1], sc[0][i]);
+                    const uint32_t w1 = pack_bf16_rne(sc[1][i - 1], sc[1][i]);
+                    pn[0][ks2][(i & 7) >> 1] = w0;
+                    pn[1][ks2][(i & 7) >> 1] = w1;
+                    psum_add(p0, bf16lo_to_f32(w0));
+                    psum_add(p1, bf16lo_to_f32(w1));
+                    psum_add(p0, bf16hi_to_f32(w0));
+                    psum_add(p1, bf16hi_to_f32(w1));
+                }
+                if (!(i & 1)) {
+                    if (i < 8) copy_one(src_k, dst_k, i >> 1);
+                    else copy_one(src_v, dst_v, (i - 8) >> 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            ps[0] = p0;
+            ps[1] = p1;
+        };
+        auto issue_copies = [&](int t) {                                 // what step t fetches
+            if (t + 3 < n_tiles) issue(Kg, lds_k + (uint32_t)(((t + 3) & 1) * PF_TILE), t + 3);
+            if (t + 2 < n_tiles) issue(Vg, lds_v + (uint32_t)(((t + 2) % 3) * PF_TILE), t + 2);
+        };
+
+        // prologue: K(0), V(0), K(1), V(1), K(2); scores and softmax of tile 0 (sets the reference),
+        // scores of tile 1.  From then on step t fetches K(t+3) and V(t+2).
+        issue(Kg, lds_k, 0);
+        issue(Vg, lds_v, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PF_LDS_BARRIER();
+        if (n_tiles > 1) {
+            issue(Kg, lds_k + PF_TILE, 1);
+            issue(Vg, lds_v + PF_TILE, 1);
+        }
+        u32x4 pa[2][2], pb[2][2], pl[2][2];
+        f32x16 sa[2], sb[2];
+        scores(0, sa, -1, -1);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            (void)sm_move_ref(c, sm_prep(0, c, sa[c]));                     // nothing accumulated yet
+            sm_finish(c, sa[c], pa[c], pl[c]);
+        }
+        if (n_tiles > 1) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            PF_LDS_BARRIER();
+            if (n_tiles > 2) issue(Kg, lds_k, 2);
+            scores(1, sa, -1, -1);
+        }
+        // now: sa = raw scores of tile t+1, pa = weights of tile t, for t = 0
+        const int d0 = (int)((first_masked_key + 1) / PF_TK);            // tiles 0 .. d0-1 need no mask
+        int t = 0;
+        bool slow = false;
+        bool top_done = false;                                           // the top of step t has been passed already
+        auto more = [&]() -> bool { return t + 1 < d0 && t + 2 < n_tiles; };
+        if (more()) {
+            step_top();
+            fetch(0, 0, 0);
+            fetch(0, 1, 1);
+            top_done = true;
+            for (;;) {
+                float ps[2];
+                pstep(t, sa, sb, pa, pb, ps);
+                if (__any(ps[0] > BIG || ps[1] > BIG)) { slow = true; break; }
+                l_part[0] += ps[0];
+                l_part[1] += ps[1];
+                t++;
+                if (!more()) {
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+                        sa[c] = sb[c];
+                        pa[c][0] = pb[c][0];
+                        pa[c][1] = pb[c][1];
+                    }
+                    break;
+                }
+                pstep(t, sb, sa, pb, pa, ps);
+                if (__any(ps[0] > BIG || ps[1] > BIG)) { slow = true; break; }
+                l_part[0] += ps[0];
+                l_part[1] += ps[1];
+                t++;
+                if (!more()) break;
+            }
+            score_done();
+        }
+        // the tiles on the diagonal and the tail, in sequence
+        if (!slow)
+            for (; t < n_tiles; t++) {
+                if (!top_done) step_top();
+                top_done = false;
+                issue_copies(t);
+                bool bad = false;
+                const float l_save[2] = {l_part[0], l_part[1]};
+                if (t + 1 < n_tiles) {
+                    const float x0 = sm_prep(t + 1, 0, sa[0]), x1 = sm_prep(t + 1, 1, sa[1]);
+                    sm_finish(0, sa[0], pb[0], pl[0]);
+                    sm_finish(1, sa[1], pb[1], pl[1]);
+                    bad = __any(x0 > m_ref[0] + SLACK || x1 > m_ref[1] + SLACK);
+                }
+                values(t, pa, pl);
+                if (bad) {
+                    l_part[0] = l_save[0];
+                    l_part[1] = l_save[1];
+                    slow = true;
+                    break;
+                }
+                if (t + 2 < n_tiles) scores(t + 2, sa, -1, -1);
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    pa[c][0] = pb[c][0];
+                    pa[c][1] = pb[c][1];
+                }
+            }
+        // slow loop (rare): entered after the top, the copies and the value products of step t; the
+        // reference follows the maximum and the accumulators are rescaled every tile
+        if (slow) {
+            bool resumed = true;
+            for (; t + 1 < n_tiles; t++) {
+                if (!resumed) {
+                    if (!top_done) step_top();
+                    top_done = false;
+                    issue_copies(t);
+                }
+                f32x16 s[2];
+                scores_global(t + 1, s);
+                float corr[2];
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    corr[c] = sm_move_ref(c, sm_prep(t + 1, c, s[c]));
+                    sm_finish(c, s[c], pb[c], pl[c]);
+                }
+                if (!resumed) values(t, pa, pl);
+                resumed = false;
+                rescale(corr);
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    pa[c][0] = pb[c][0];
+                    pa[c][1] = pb[c][1];
+                }
+            }
+            if (!top_done) step_top();
+            values(n_tiles - 1, pa, pl);
+        }
     }
-    // ---- last tile's values ----
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    PF_LDS_BARRIER();
-    values(n_tiles - 1, pw, pl);
 
     // ---- epilogue ----
 #pragma unroll
@@ -413,11 +653,23 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
                    const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
                    float scale_log2e, float *__restrict__ out, int64_t n_prec) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    // heavy (late) position blocks first, over all kv heads: workgroups are handed out in grid
-    // order, and under the causal triangle the last ones to start must be the short ones
+    // Workgroups are handed out in grid order, so the grid runs from the most expensive position
+    // block to the cheapest (the last ones to start must be the short ones).  A block costs its
+    // number of key tiles, and 1.6 times that in the PRECISE variant: rank r = blockIdx.x /
+    // n_kv_heads in the merge of the two descending sequences 10 (p+1), p >= n_prec, and
+    // 16 (p+1), p < n_prec.
     const int64_t pblocks = (int64_t)gridDim.x / n_kv_heads;
-    const int64_t pblk = pblocks - 1 - (int64_t)blockIdx.x / n_kv_heads;
+    const int64_t rank = (int64_t)blockIdx.x / n_kv_heads;
     const int kvh = (int)(blockIdx.x % n_kv_heads);
+    int64_t pblk = -1, before = 0;                      // precise blocks ranked before this one
+    for (int64_t pp = n_prec - 1; pp >= 0; pp--) {
+        int64_t qmin = 16 * (pp + 1) / 10;              // plain blocks q >= qmin cost more than precise block pp
+        if (qmin < n_prec) qmin = n_prec;
+        const int64_t rk = (qmin < pblocks ? pblocks - qmin : 0) + (n_prec - 1 - pp);
+        if (rk == rank) pblk = pp;
+        if (rk < rank) before++;
+    }
+    if (pblk < 0) pblk = pblocks - 1 - (rank - before);
     if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
     else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
 }

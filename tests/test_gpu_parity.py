@@ -71,6 +71,11 @@ def test_gqa_decode(hip, orc, n_keys, nh, nkv, hd):
     (0, 130, 8, 8),          # group 1
     (5, 200, 16, 2),         # group 8
     (0, 64, 4, 2),           # group 2
+    # beyond 2048 keys the kernel leaves its two-term-weight variant for the pipelined one:
+    (2100, 150, 16, 4),      # every position block on the long-prefix path, ragged tiles
+    (0, 2300, 8, 2),         # one launch that crosses the boundary between the two variants
+    (1990, 200, 4, 4),       # the boundary inside a chunk, group 1
+    (3000, 40, 16, 2),       # group 8, a chunk shorter than one position block
 ])
 def test_gqa_prefill(hip, orc, pos0, n, nh, nkv):
     say("[case] gqa_prefill", pos0, n, nh, nkv)
@@ -87,22 +92,37 @@ def test_gqa_prefill(hip, orc, pos0, n, nh, nkv):
     cache.free()
 
 
-def test_gqa_prefill_growing_scores(hip, orc):
+@pytest.mark.parametrize("pos0,n,start,slope", [
+    (0, 300, 0, 0.5),        # short prefix: the two-term-weight variant
+    # long prefix: the pipelined variant leaves its fast loop after a few steps / after many.
+    # The slope is smaller there so that the raw scores stay below 2e4 as in the first case:
+    # fp32 dot products of 1e5 differ by 1e-3 in the exponent between summation orders.
+    (2100, 150, 0, 0.05),
+    (2100, 150, 1100, 0.1),
+])
+def test_gqa_prefill_growing_scores(hip, orc, pos0, n, start, slope):
     """Scores that climb by far more than 2^64 along the keys: the rows must leave the fixed
     softmax reference of their first tile and follow the maximum (rescaling path)."""
-    say("[case] gqa_prefill growing scores")
-    n, nh, nkv = 300, 16, 4
-    c = synth.cfg2_gqa_prefill(n, nh, nkv, 256, 0, seed=777)
-    k = synth.bf16_to_f32(c["k"]).reshape(n, nkv, 256)
+    say("[case] gqa_prefill growing scores", pos0, n, start, slope)
+    nh, nkv = 16, 4
+    nk = pos0 + n
+    c = synth.cfg2_gqa_prefill(n, nh, nkv, 256, pos0, seed=777)
+    k = synth.bf16_to_f32(c["k"]).reshape(nk, nkv, 256)
     q = synth.bf16_to_f32(c["q"]).reshape(n, nh, 256)
-    # a common direction whose weight grows with the key index: q.k gains about i * 4 per key
-    k[:, :, 0] = np.arange(n, dtype=np.float32)[:, None] * 0.5
-    q[:, :, 0] = 8.0 * 16.0                                   # times scale 1/16 -> 8 * 0.5 * i
-    ck = synth.f32_to_bf16(k.reshape(n, -1)); cq = synth.f32_to_bf16(q.reshape(n, nh, 256))
-    cache = hip.KVCache(n, nkv, 256)
-    cache.write(0, ck, c["v"].reshape(n, -1))
-    got = hip.gqa_prefill(cache, 0, cq, c["scale"])
-    ref = orc.gqa_prefill(cq, ck.reshape(n, nkv, 256), c["v"], 0, c["scale"], nthreads=0)
+    # a common direction whose weight grows with the key index: q.k gains 8 * slope per key
+    k[:, :, 0] = np.maximum(np.arange(nk, dtype=np.float32) - start, 0.0)[:, None] * slope
+    q[:, :, 0] = 8.0 * 16.0                                   # times scale 1/16 -> 8 * slope * i
+    ck = synth.f32_to_bf16(k.reshape(nk, -1)); cq = synth.f32_to_bf16(q.reshape(n, nh, 256))
+    cv = c["v"]
+    if pos0 + n > 2048:
+        # Beyond 2048 keys the weights are single bf16 terms: a softmax that a handful of keys
+        # share, as here, is off by 2^-9 of the spread of their values.  Values within +-1.2
+        # keep that inside the tolerance; the case is about the moving reference.
+        cv = synth.f32_to_bf16(synth.bf16_to_f32(cv) * 0.25)
+    cache = hip.KVCache(nk, nkv, 256)
+    cache.write(0, ck, cv.reshape(nk, -1))
+    got = hip.gqa_prefill(cache, pos0, cq, c["scale"])
+    ref = orc.gqa_prefill(cq, ck.reshape(nk, nkv, 256), cv, pos0, c["scale"], nthreads=0)
     assert np.isfinite(got).all()
     assert_close(got, ref, "gqa_prefill growing scores", strict=False)
     cache.free()
