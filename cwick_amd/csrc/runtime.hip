@@ -788,7 +788,7 @@ int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches) {
 const char *cwick_hip_prof_name(int which) {
     static const char *names[CWICK_HIP_PROF_COUNT] = {
         "gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk_radix_reg_kernel"};
+        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk kernels"};
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 

@@ -291,12 +291,254 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     }
 }
 
+// ---- rows of 16 K .. 128 K scores: many workgroups per row ----
+// One workgroup of TOPK_MW_THREADS takes TOPK_MW_KEYS consecutive scores, so a batch of eight
+// 64 K rows fills the chip instead of eight CUs.  Workgroups of a row meet only at kernel
+// boundaries: kernel p (p = 0..3) counts the p-th digit of the keys that match the digits
+// chosen so far into the workgroup's own 256-bin slice (no atomics across workgroups, nothing
+// to clear), and every workgroup of kernel p+1 first adds up the slices of its row and picks
+// digit p exactly as the single-workgroup kernels do.  The last kernel knows T and the tie
+// budget r, derives the output offset of its workgroup from the slices (the keys above T of
+// an earlier workgroup are those that left the chosen path at some digit with a larger bin)
+// and writes its indices in ascending order.
+constexpr int TOPK_MW_THREADS = 256;
+constexpr int TOPK_MW_EPT = 8;
+constexpr int TOPK_MW_KEYS = TOPK_MW_THREADS * TOPK_MW_EPT;     // 2048
+constexpr int TOPK_MW_MAX_WGS = 64;                              // per row
+
+struct TopkMwState { uint32_t prefix, remaining; };
+
+// sum of p[w * 256] over w < count with sixteen loads in flight (the slices sit in L2: a
+// dependent chain of loads would cost a round trip each)
+__device__ __forceinline__ uint32_t topk_mw_colsum(const uint32_t *__restrict__ p, int count) {
+    uint32_t c = 0u;
+    for (int w0 = 0; w0 < count; w0 += 16) {
+        uint32_t v[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = w0 + j < count ? p[(size_t)(w0 + j) * 256] : 0u;
+#pragma unroll
+        for (int j = 0; j < 16; j++) c += v[j];
+    }
+    return c;
+}
+
+// adds up the slices of pass p of this row, picks the digit that holds the remaining-th best
+// key; all threads return the new (prefix, remaining)
+__device__ __forceinline__ TopkMwState
+topk_mw_pick(const uint32_t *__restrict__ slices, int n_wg, int shift, TopkMwState st,
+             uint32_t *hist /* LDS, 256 */, TopkMwState *sh_state /* LDS */) {
+    const int tid = threadIdx.x;
+    hist[tid] = topk_mw_colsum(slices + tid, n_wg);
+    __syncthreads();
+    if (tid < 64) {
+        // walk the 256 buckets from the largest digit down; lane b owns buckets 255-4b .. 252-4b
+        uint32_t cc[4], sum = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            cc[j] = hist[255 - (tid * 4 + j)];
+            sum += cc[j];
+        }
+        uint32_t inc = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t t = __shfl_up(inc, o, 64);
+            if (tid >= o) inc += t;
+        }
+        uint32_t before = inc - sum;       // elements in strictly larger buckets
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (before < st.remaining && st.remaining <= before + cc[j]) {
+                sh_state->prefix = st.prefix | ((uint32_t)(255 - (tid * 4 + j)) << shift);
+                sh_state->remaining = st.remaining - before;
+            }
+            before += cc[j];
+        }
+    }
+    __syncthreads();
+    const TopkMwState out = *sh_state;
+    __syncthreads();
+    return out;
+}
+
+// workspace of a row: slices[4][n_wg][256], then state[4]
+__global__ void __launch_bounds__(TOPK_MW_THREADS)
+topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int n_wg, int pass,
+                    uint32_t *__restrict__ ws, size_t ws_row) {
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t hist8[256 * 8];
+    __shared__ TopkMwState sh_state;
+    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x;
+    uint32_t *slices = ws + (size_t)row * ws_row;
+    TopkMwState *state = (TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    const int64_t kk = k < n ? k : n;
+    // the workgroup's scores: issued first, they travel while the previous digit is picked
+    const float *sc = scores + (size_t)row * n;
+    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
+    float v[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        v[j] = i < n ? sc[i] : 0.0f;
+    }
+    TopkMwState st{0u, (uint32_t)kk};
+    if (pass > 0) {
+        if (pass > 1) st = state[pass - 1];
+        st = topk_mw_pick(slices + (size_t)(pass - 1) * n_wg * 256, n_wg, 32 - 8 * pass, st, hist, &sh_state);
+        if (wg == 0 && tid == 0) state[pass] = st;
+    }
+    const int shift = 24 - 8 * pass;
+    const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (32 - 8 * pass));
+#pragma unroll
+    for (int j = 0; j < 8; j++) hist8[tid + 256 * j] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        if (i < n) {
+            const uint32_t key = topk_key(v[j]);
+            // eight copies picked by lane: scores cluster in a few buckets and same-address
+            // LDS atomics of one instruction serialise
+            if ((key & mask) == st.prefix) atomicAdd(&hist8[((key >> shift) & 0xFFu) * 8 + (tid & 7)], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t c = 0u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) c += hist8[tid * 8 + ((j + tid) & 7)];
+    slices[((size_t)pass * n_wg + wg) * 256 + tid] = c;
+}
+
+__global__ void __launch_bounds__(TOPK_MW_THREADS)
+topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
+                    const uint32_t *__restrict__ ws, size_t ws_row, int32_t *__restrict__ out) {
+    __shared__ uint32_t hist[256];
+    __shared__ TopkMwState sh_state;
+    __shared__ uint32_t sh_red[2][TOPK_MW_THREADS / 64];
+    __shared__ uint32_t sh_gt[TOPK_MW_EPT][TOPK_MW_THREADS / 64], sh_eq[TOPK_MW_EPT][TOPK_MW_THREADS / 64];
+    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t *slices = ws + (size_t)row * ws_row;
+    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    int32_t *dst = out + (size_t)row * k;
+    const int64_t kk = k < n ? k : n;
+    if (wg == 0)
+        for (int64_t i = kk + tid; i < k; i += TOPK_MW_THREADS) dst[i] = -1;
+    const float *sc = scores + (size_t)row * n;
+    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
+    uint32_t keys[TOPK_MW_EPT];                 // issued first: they travel while T is picked
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        keys[j] = i < n ? topk_key(sc[i]) : 0u;
+    }
+    // keys above T in the workgroups before this one, part 1: bin `tid` of pass p of workgroup w
+    // counts keys that match the chosen digits 0..p-1 and have digit p = tid; they are above T
+    // if tid is larger than the chosen digit p.  Digits 0..2 are known before the last pick:
+    // their loads go out together and travel while it runs.
+    const TopkMwState st3 = state[3];
+    uint32_t gt = 0u, eq = 0u;
+    {
+        bool above[3];
+#pragma unroll
+        for (int p = 0; p < 3; p++) above[p] = (uint32_t)tid > ((st3.prefix >> (24 - 8 * p)) & 0xFFu);
+        for (int w0 = 0; w0 < wg; w0 += 8) {
+            uint32_t v[3][8];
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    v[p][j] = (above[p] && w0 + j < wg) ? slices[((size_t)p * n_wg + w0 + j) * 256 + tid] : 0u;
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) gt += v[p][j];
+        }
+    }
+    const TopkMwState st = topk_mw_pick(slices + (size_t)3 * n_wg * 256, n_wg, 0, st3, hist, &sh_state);
+    const uint32_t T = st.prefix, r = st.remaining;   // r ties belong to the selection
+    {   // part 2: the last digit; equal to T if it is the digit itself
+        const uint32_t dig = T & 0xFFu;
+        const bool above = (uint32_t)tid > dig, same = (uint32_t)tid == dig;
+        const uint32_t c = topk_mw_colsum(slices + (size_t)3 * n_wg * 256 + tid, (above || same) ? wg : 0);
+        if (above) gt += c;
+        if (same) eq += c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        gt += __shfl_xor(gt, o, 64);
+        eq += __shfl_xor(eq, o, 64);
+    }
+    if (lane == 0) {
+        sh_red[0][wave] = gt;
+        sh_red[1][wave] = eq;
+    }
+    // own keys, in index order: element (j, tid) is index base + 256 j + tid, so the order of
+    // the workgroup is (j, wave, lane).  Ballots give the counts of every (j, wave) cell, one
+    // walk over the 32 cells the position of this wave's cells.
+    uint64_t m_gt[TOPK_MW_EPT], m_eq[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        m_gt[j] = __ballot(i < n && keys[j] > T);
+        m_eq[j] = __ballot(i < n && keys[j] == T);
+        if (lane == 0) {
+            sh_gt[j][wave] = (uint32_t)__builtin_popcountll(m_gt[j]);
+            sh_eq[j][wave] = (uint32_t)__builtin_popcountll(m_eq[j]);
+        }
+    }
+    __syncthreads();
+    uint32_t gt_before = 0u, eq_before = 0u;
+#pragma unroll
+    for (int w = 0; w < TOPK_MW_THREADS / 64; w++) {
+        gt_before += sh_red[0][w];
+        eq_before += sh_red[1][w];
+    }
+    uint32_t run_pos = gt_before + (eq_before < r ? eq_before : r), run_eq = eq_before;
+    uint32_t my_pos[TOPK_MW_EPT], my_eq[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++)
+#pragma unroll
+        for (int w = 0; w < TOPK_MW_THREADS / 64; w++) {
+            const uint32_t g = sh_gt[j][w], e = sh_eq[j][w];
+            if (w == wave) {
+                my_pos[j] = run_pos;
+                my_eq[j] = run_eq;
+            }
+            run_pos += g + (run_eq >= r ? 0u : (r - run_eq < e ? r - run_eq : e));
+            run_eq += e;
+        }
+    const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        const bool is_gt = (m_gt[j] >> lane) & 1, is_eq = (m_eq[j] >> lane) & 1;
+        // ties first get their rank, then every taken element its slot
+        const uint32_t my_eq_rank = my_eq[j] + (uint32_t)__builtin_popcountll(m_eq[j] & lt);
+        const bool take = is_gt || (is_eq && my_eq_rank < r);
+        const uint64_t m_take = __ballot(take);
+        if (take) dst[my_pos[j] + (uint32_t)__builtin_popcountll(m_take & lt)] = (int32_t)i;
+    }
+}
+
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s) {
     CWICK_REQUIRE(scores && out_idx, "topk: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 65535, "topk: batch %d", batch);
     CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
+    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
+    if (n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS) {
+        const size_t ws_row = (size_t)4 * n_wg * 256 + 2 * 4;       // dwords: slices, then four states
+        uint32_t *ws = (uint32_t *)workspace(s, (size_t)batch * ws_row * sizeof(uint32_t));
+        CWICK_REQUIRE(ws, "topk: workspace allocation failed");
+        const dim3 grid((unsigned)n_wg, (unsigned)batch);
+        ProfScope ps(CWICK_HIP_PROF_TOPK, s);
+        for (int pass = 0; pass < 4; pass++)
+            topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row);
+        topk_mw_emit_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, out_idx);
+        CWICK_HIP_CALL(hipGetLastError());
+        return 1;
+    }
     {
         ProfScope ps(CWICK_HIP_PROF_TOPK, s);
         if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)

@@ -404,7 +404,7 @@ def dsa_decode_dev(ikeys, ikscale, key_bstride, kscale_bstride, rows, scales, ro
 
 # ------------------------------------------------------------------ phase timers
 PROF_NAMES = ["gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk_radix_reg_kernel"]
+              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk kernels"]
 
 
 def prof_enable(on=True):

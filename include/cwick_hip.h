@@ -256,7 +256,7 @@ enum {
     CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill) */
     CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag16_kernel after it */
     CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel */
-    CWICK_HIP_PROF_TOPK,                /* topk_radix_reg_kernel / topk_radix_kernel */
+    CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel */
     CWICK_HIP_PROF_COUNT
 };
 void cwick_hip_prof_enable(int on);

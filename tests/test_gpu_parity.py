@@ -240,6 +240,11 @@ def test_topk_known_answers(hip, orc, sc, k, want):
     (65536, 2048, "normal"), (65536, 2048, "ties"), (65536, 2048, "const"),
     (100000, 512, "normal"), (5000, 5000, "normal"), (3000, 4096, "ties"),
     (1 << 20, 2048, "ties"), (777, 1, "normal"), (4097, 2048, "inf"),
+    # 16 K .. 128 K scores take the many-workgroup kernels:
+    (40000, 1000, "ties"),           # ragged last workgroup, ties across workgroup borders
+    (131072, 70, "const"),           # the largest such row; every score ties
+    (16384, 16384, "normal"),        # the smallest; k = n
+    (20000, 4096, "inf"), (131073, 2048, "normal"),
 ])
 def test_topk_bit_exact(hip, orc, n, k, kind):
     say("[case] topk", n, k, kind)
@@ -258,18 +263,22 @@ def test_topk_bit_exact(hip, orc, n, k, kind):
     assert np.array_equal(got, ref)
 
 
-def test_dsa_decode_small(hip, orc):
-    say("[case] dsa_decode small")
-    c = synth.cfg5_dsa(n_keys=3000, batch=3, ih=64, topk=256, nh=128, seed=909)
-    ik = hip.IndexKeys(3, 3000)
-    lat = hip.LatentCache(3, 3000)
+@pytest.mark.parametrize("n_keys,topk", [
+    (3000, 256),         # one workgroup per query in the top-k
+    (20000, 512),        # many workgroups per query, batched
+])
+def test_dsa_decode_small(hip, orc, n_keys, topk):
+    say("[case] dsa_decode small", n_keys, topk)
+    c = synth.cfg5_dsa(n_keys=n_keys, batch=3, ih=64, topk=topk, nh=128, seed=909)
+    ik = hip.IndexKeys(3, n_keys)
+    lat = hip.LatentCache(3, n_keys)
     for b in range(3):
         ik.write(b, 0, c["ikeys"][b], c["ikscale"][b])
         lat.write(b, 0, c["rows"][b], c["scales"][b])
-    out, sel = hip.dsa_decode(ik, lat, 0, 1, 3000, c["q_idx"], c["w"], 256, c["q"], c["scale"])
+    out, sel = hip.dsa_decode(ik, lat, 0, 1, n_keys, c["q_idx"], c["w"], topk, c["q"], c["scale"])
     for b in range(3):
         sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], c["ikeys"][b], c["ikscale"][b], nthreads=0)
-        rsel = orc.topk_contract(sc, 256)
+        rsel = orc.topk_contract(sc, topk)
         assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
         ref = orc.mla_decode(c["q"][b], c["rows"][b], c["scales"][b], c["scale"], sel=rsel, nthreads=0)
         assert_close(out[b], ref, "dsa_decode query %d" % b)
