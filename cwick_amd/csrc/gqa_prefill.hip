@@ -38,7 +38,7 @@
 //   to 2^64 lose nothing in bf16 or fp32.  A wave that meets a larger score
 //   leaves the fast loop for a slow one that moves the reference and rescales
 //   the accumulators (in place, in AGPRs) every tile.
-//   Position blocks that see at most 2048 keys run the PRECISE variant (the
+//   Position blocks that see at most 1024 keys run the PRECISE variant (the
 //   rounding residual of the weights goes through the matrix core too) in the
 //   simpler two-stage schedule: scores of tile t+1, then its softmax next to
 //   the value products of tile t.
@@ -76,7 +76,7 @@ struct PfSmem {
 #define PF_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 // PRECISE: the bf16 rounding residual of the weights goes through the matrix core as well
-// (position blocks that see at most 2048 keys; see the launcher).  The body of one workgroup:
+// (position blocks that see at most 1024 keys; see the launcher).  The body of one workgroup:
 template <int GROUP, bool PRECISE>
 __device__ __forceinline__ void
 gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
@@ -674,6 +674,17 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
 }
 
+// rows that see at most this many keys take the two-term-weight variant
+static int64_t gqa_precise_keys() {
+    static int64_t v = -1;
+    if (v < 0) {
+        const char *e = getenv("CWICK_HIP_GQA_PRECISE_KEYS");
+        v = e ? atoll(e) : 1024;
+        if (v < 0) v = 0;
+    }
+    return v;
+}
+
 template <int GROUP>
 static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
                            int n_kv_heads, const uint16_t *q, float scale, float *out,
@@ -689,13 +700,13 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     const int64_t pblocks = (n + P - 1) / P;
     CWICK_REQUIRE(pblocks * n_kv_heads <= 0x7FFFFFFF, "gqa_prefill: grid too large");
     // Short prefixes: few keys carry the whole weight, so the 2^-9 rounding of each bf16 weight
-    // shows in an O(1) output.  Position blocks that see at most 2048 keys run the variant that
+    // shows in an O(1) output.  Position blocks that see at most 1024 keys run the variant that
     // also feeds the rounding residual through the matrix core (weights good to 2^-17).
     int64_t n_prec = 0;
     while (n_prec < pblocks) {
         int64_t last_t = (n_prec + 1) * P - 1;
         if (last_t > n - 1) last_t = n - 1;
-        if (pos0 + last_t + 1 > 2048) break;
+        if (pos0 + last_t + 1 > gqa_precise_keys()) break;
         n_prec++;
     }
     {

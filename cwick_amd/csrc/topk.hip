@@ -13,8 +13,11 @@
 //   2. one ordered pass emits every index with key > T and the first r indices
 //      with key == T, in ascending index order, through a block-wide scan.
 //
-// One workgroup of 1024 threads per batch row.  Rows of up to 65536 scores (the
-// indexer's case) are read once: every thread keeps its 64 consecutive keys in
+// Rows of 16 K to 128 K scores (the indexer's case) are split over many
+// workgroups that meet at kernel boundaries: four digit-histogram launches and
+// one ordered emit (see topk_mw_hist_kernel below).  Other rows take one
+// workgroup of 1024 threads.  Up to 65536 scores
+// are read once: every thread keeps its 64 consecutive keys in
 // registers for all five passes, the first histogram pass counts into one of 32
 // lane-indexed copies (scores cluster in a few exponent buckets, and same-address
 // LDS atomics serialise), and the ordered emit places elements with ballots

@@ -71,10 +71,11 @@ def test_gqa_decode(hip, orc, n_keys, nh, nkv, hd):
     (0, 130, 8, 8),          # group 1
     (5, 200, 16, 2),         # group 8
     (0, 64, 4, 2),           # group 2
-    # beyond 2048 keys the kernel leaves its two-term-weight variant for the pipelined one:
+    # beyond 1024 keys the kernel leaves its two-term-weight variant for the pipelined one:
     (2100, 150, 16, 4),      # every position block on the long-prefix path, ragged tiles
     (0, 2300, 8, 2),         # one launch that crosses the boundary between the two variants
-    (1990, 200, 4, 4),       # the boundary inside a chunk, group 1
+    (1990, 200, 4, 4),       # group 1
+    (1000, 100, 8, 4),       # the boundary between the variants inside a chunk
     (3000, 40, 16, 2),       # group 8, a chunk shorter than one position block
 ])
 def test_gqa_prefill(hip, orc, pos0, n, nh, nkv):
@@ -114,8 +115,8 @@ def test_gqa_prefill_growing_scores(hip, orc, pos0, n, start, slope):
     q[:, :, 0] = 8.0 * 16.0                                   # times scale 1/16 -> 8 * slope * i
     ck = synth.f32_to_bf16(k.reshape(nk, -1)); cq = synth.f32_to_bf16(q.reshape(n, nh, 256))
     cv = c["v"]
-    if pos0 + n > 2048:
-        # Beyond 2048 keys the weights are single bf16 terms: a softmax that a handful of keys
+    if pos0 + n > 1024:
+        # Beyond 1024 keys the weights are single bf16 terms: a softmax that a handful of keys
         # share, as here, is off by 2^-9 of the spread of their values.  Values within +-1.2
         # keep that inside the tolerance; the case is about the moving reference.
         cv = synth.f32_to_bf16(synth.bf16_to_f32(cv) * 0.25)
