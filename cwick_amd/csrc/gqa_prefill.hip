@@ -134,10 +134,12 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     const uint16_t *Vg = V + (size_t)kvh * PF_HD + 8 * g;
     const uint32_t lds_k = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.k[0][0];
     const uint32_t lds_v = (uint32_t)(uintptr_t)(pf_lds_void *)&sm.v[0][0];
+    // (32-bit row arithmetic: at most 2^30 keys, and a row of at most 64 kv heads)
+    const uint32_t last_key = (uint32_t)(n_keys_all - 1), kv_stride32 = (uint32_t)kv_stride;
     auto copy_src = [&](const uint16_t *base, int tile) -> const uint16_t * {
-        int64_t row = (int64_t)tile * PF_TK + cp_key;
-        if (row > n_keys_all - 1) row = n_keys_all - 1;         // masked anyway
-        return base + row * kv_stride + 64 * wave;
+        uint32_t row = (uint32_t)tile * PF_TK + (uint32_t)cp_key;
+        row = row < last_key ? row : last_key;                  // masked anyway
+        return base + (uint64_t)row * kv_stride32 + 64 * wave;
     };
     auto copy_one = [&](const uint16_t *src, uint32_t lds_tile, int i) {      // block 4 wave + i
         const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK));
@@ -439,9 +441,12 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
         constexpr float BIG = 18446744073709551616.0f;                  // 2^SLACK
         u32x4 ka[2], qa[2];                                             // fragments of the next two slots
         s16x4 lo[2], hi[2];
-        auto fetch = [&](int t, int i, int slot) {                      // fragments of slot i of step t
+        // V(t) lives in buffer t mod 3, carried along as t3 (no division in the loop)
+        auto next3 = [](int x) -> int { return x == 2 ? 0 : x + 1; };
+        int t3 = 0;
+        auto fetch = [&](int t, int t3, int i, int slot) {              // fragments of slot i of step t
             const unsigned char *kb = &sm.k[t & 1][0] + kfrag_off;      // K(t+2)
-            const unsigned char *vb = &sm.v[t % 3][0];                  // V(t)
+            const unsigned char *vb = &sm.v[t3][0];                     // V(t)
             ka[slot] = *(const u32x4 *)(kb + i * PF_BLK);
             if (i >= PF_QX0) qa[slot] = sm.qx[wave][i - PF_QX0][lane];
             const int ks2 = i >> 3, db = i & 7;
@@ -451,12 +456,11 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
         // the running sums as opaque instructions: left to the compiler, the thirty-two additions
         // of a step sink to its end, a dependent chain behind the last MFMA
         auto psum_add = [&](float &acc, float x) { asm volatile("v_add_f32 %0, %1, %0" : "+v"(acc) : "v"(x)); };
-        auto pstep = [&](int t, f32x16 (&sc)[2], f32x16 (&sn)[2], const u32x4 (&pc)[2][2],
+        auto pstep = [&](int t, int t3, f32x16 (&sc)[2], f32x16 (&sn)[2], const u32x4 (&pc)[2][2],
                          u32x4 (&pn)[2][2], float (&ps)[2]) {
-            const uint16_t *src_k = copy_src(Kg, t + 3);     // past the last tile: clipped rows into a dead buffer
-            const uint16_t *src_v = copy_src(Vg, t + 2);
-            const uint32_t dst_k = lds_k + (uint32_t)(((t + 1) & 1) * PF_TILE);
-            const uint32_t dst_v = lds_v + (uint32_t)(((t + 2) % 3) * PF_TILE);
+            const int t3n = next3(t3);
+            const uint16_t *src_k = nullptr, *src_v = nullptr;
+            uint32_t dst_k = 0, dst_v = 0;
             const float mu0 = m_ref[0], mu1 = m_ref[1];
             float p0 = 0.0f, p1 = 0.0f;
 #pragma unroll
@@ -468,6 +472,14 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                 const bf16x8 va = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo[i & 1], hi[i & 1], 0, 1, 2, 3, 4, 5, 6, 7));
                 score_mfma(sn[0], kf, qf[0][i], i == 0);
                 sc[0][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][i], scale_log2e, -mu0));
+                if (i == 0) {
+                    // where this step's copies come from and go to, worked out behind the
+                    // first MFMA (past the last tile: clipped rows into a dead buffer)
+                    src_k = copy_src(Kg, t + 3);
+                    src_v = copy_src(Vg, t + 2);
+                    dst_k = lds_k + (uint32_t)(((t + 1) & 1) * PF_TILE);
+                    dst_v = lds_v + (uint32_t)(next3(t3n) * PF_TILE);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 oacc[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pc[0][ks2]), oacc[0][db], 0, 0, 0);
                 sc[1][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[1][i], scale_log2e, -mu1));
@@ -478,8 +490,8 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                     asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
                     PF_LDS_BARRIER();
                 }
-                if (i < 14) fetch(t, i + 2, i & 1);
-                else fetch(t + 1, i - 14, i & 1);
+                if (i < 14) fetch(t, t3, i + 2, i & 1);
+                else fetch(t + 1, t3n, i - 14, i & 1);
                 __builtin_amdgcn_sched_barrier(0);
                 oacc[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, __builtin_bit_cast(bf16x8, pc[1][ks2]), oacc[1][db], 0, 0, 0);
                 if (i & 1) {                                         // weights, and the sum of the rounded weights
@@ -538,16 +550,17 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
         auto more = [&]() -> bool { return t + 1 < d0 && t + 2 < n_tiles; };
         if (more()) {
             step_top();
-            fetch(0, 0, 0);
-            fetch(0, 1, 1);
+            fetch(0, 0, 0, 0);
+            fetch(0, 0, 1, 1);
             top_done = true;
             for (;;) {
                 float ps[2];
-                pstep(t, sa, sb, pa, pb, ps);
+                pstep(t, t3, sa, sb, pa, pb, ps);
                 if (__any(ps[0] > BIG || ps[1] > BIG)) { slow = true; break; }
                 l_part[0] += ps[0];
                 l_part[1] += ps[1];
                 t++;
+                t3 = next3(t3);
                 if (!more()) {
 #pragma unroll
                     for (int c = 0; c < 2; c++) {
@@ -557,11 +570,12 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                     }
                     break;
                 }
-                pstep(t, sb, sa, pb, pa, ps);
+                pstep(t, t3, sb, sa, pb, pa, ps);
                 if (__any(ps[0] > BIG || ps[1] > BIG)) { slow = true; break; }
                 l_part[0] += ps[0];
                 l_part[1] += ps[1];
                 t++;
+                t3 = next3(t3);
                 if (!more()) break;
             }
             score_done();
