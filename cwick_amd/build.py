@@ -17,14 +17,14 @@ OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libcwick_hip.so")
 
 SOURCES = ["runtime.hip", "misc.hip", "gqa_decode.hip", "gqa_prefill.hip", "mla.hip",
-           "mla_stream.hip", "mla_dsplit.hip", "mla_roles.hip", "indexer.hip", "topk.hip"]
+           "mla_stream.hip", "mla_dsplit.hip", "mla_roles.hip", "indexer.hip", "indexer_band.hip", "topk.hip"]
 
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
           "-Wall", "-Wno-unused-function",
           # packed-fp32 VALU forms are kept out of every kernel in this library
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # the indexer's summation order is a contract: nothing may be fused behind its back
-PER_FILE = {"indexer.hip": ["-ffp-contract=off"]}
+PER_FILE = {"indexer.hip": ["-ffp-contract=off"], "indexer_band.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc():

@@ -64,6 +64,34 @@ int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_
                           int64_t kscale_bstride, int batch, int64_t n_keys,
                           const uint16_t *q_idx, const float *w, int n_idx_heads,
                           float *scores, hipStream_t s);
+// ---- fused select: approximate scores with an error band, exact scores for the keys inside it
+// (indexer_band.hip).  One of these per batch row, in the workspace:
+struct IndexerBandRow {
+    uint32_t n_cand;      // keys inside the band (may exceed the list's capacity)
+    uint32_t fallback;    // the band could not be formed (bound not finite, NaN threshold)
+};
+constexpr int CWICK_INDEXER_BAND_CAP = 4096;   // candidate list entries per row
+__host__ __device__ inline bool indexer_band_failed(const IndexerBandRow &r, int cap) {
+    return r.fallback != 0u || r.n_cand > (uint32_t)cap;
+}
+// shapes the banded path takes: rows that the many-workgroup top-k handles, k < n
+inline bool indexer_band_applies(int64_t n_keys, int64_t k, int n_idx_heads) {
+    return n_keys >= 16384 && n_keys <= 131072 && k < n_keys && n_idx_heads >= 1 && n_idx_heads <= 64;
+}
+int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                          int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
+                          const float *w, int n_idx_heads, int64_t k, float *scores, hipStream_t s);
+// the exact kernel for the rows whose band failed (returns at once for the others)
+int launch_indexer_scores_rows(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                               int64_t kscale_bstride, int batch, int64_t n_keys,
+                               const uint16_t *q_idx, const float *w, int n_idx_heads, float *scores,
+                               const IndexerBandRow *rows, int cap, hipStream_t s);
+// top-k machinery on approximate scores: finds T, then patches the scores (+inf / -inf / kept)
+// and lists the keys within 2 beta of T.  `ws` holds topk_mw_workspace_bytes() at its start.
+size_t topk_mw_workspace_bytes(int batch, int64_t n);
+int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
+                              const float *beta_slots, int n_beta, int32_t *cand, int cap,
+                              IndexerBandRow *rows, hipStream_t s);
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s);
 int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,

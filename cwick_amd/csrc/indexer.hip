@@ -41,8 +41,11 @@ indexer_scores_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
                       const uint16_t *__restrict__ q,  // [batch][ih][128] bf16
                       const float *__restrict__ w,     // [batch][ih]
-                      int ih, float *__restrict__ scores) {
+                      int ih, float *__restrict__ scores,
+                      const IndexerBandRow *__restrict__ rows, int cap) {
     const int b = blockIdx.y;
+    // after a banded select: only the rows whose band failed are computed
+    if (rows && !indexer_band_failed(rows[b], cap)) return;
     const int64_t t = (int64_t)blockIdx.x * IDX_THREADS + threadIdx.x;
     const bool live = t < n_keys;
     const int64_t tc = live ? t : n_keys - 1;
@@ -145,8 +148,20 @@ int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_
     {
         ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
         indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
-                                                           n_keys, q_idx, w, n_idx_heads, scores);
+                                                           n_keys, q_idx, w, n_idx_heads, scores, nullptr, 0);
     }
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_indexer_scores_rows(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                               int64_t kscale_bstride, int batch, int64_t n_keys,
+                               const uint16_t *q_idx, const float *w, int n_idx_heads, float *scores,
+                               const IndexerBandRow *rows, int cap, hipStream_t s) {
+    CWICK_REQUIRE(rows, "indexer_scores_rows: null pointer");
+    dim3 grid((unsigned)((n_keys + IDX_THREADS - 1) / IDX_THREADS), batch);
+    indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
+                                                       n_keys, q_idx, w, n_idx_heads, scores, rows, cap);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -1,0 +1,325 @@
+// indexer_band.hip -- the indexer scores of a fused select (indexer -> top-k) without running
+// the exact vector-ALU kernel over every key.
+//
+// The selection has to be the one the reference makes (src/attention.c:573-598,
+// src/ds_model.c:1108-1152): bit-identical scores for every key that could change it.  Most
+// keys cannot.  So:
+//
+//   1. indexer_approx_kernel: approximate scores on the bf16 matrix cores,
+//          st[t] = ks[t] * sum_h w[h] * max(q_h . e_t, 0),
+//      and next to them a bound on |st[t] - s[t]|, s the reference's score.  The products
+//      e*q are exact in fp32 either way (a 4-bit times an 8-bit significand); the two sides
+//      differ in the order of the additions and in a handful of roundings:
+//          reference dot (dot_f32: four fma chains of 32, three additions)  35 roundings
+//          matrix-core dot, any order and any internal truncation          <= 256 roundings
+//          scale, weight, sum over at most 64 heads, on each side          <= 2 * 66 roundings
+//      each relative to A_h = sum_i |e_i||q_hi| >= |q_h . e_t|, so
+//          |st - s| <= 450 u * ks[t] * sum_h |w_h| A_h[t],   u = 2^-24,
+//      and sum_h |w_h| A_h[t] = sum_i |e_ti| c_i with c_i = sum_h |w_h||q_hi|: one more row
+//      through the matrix core, with c rounded up to bf16.  beta[t] = 512 u * ks[t] * that row
+//      (the slack covers the rounding of the bound itself); beta = max_t beta[t].
+//   2. top-k machinery on st: T = the k-th largest approximate score (topk.hip).
+//   3. classify: at most k-1 keys have st > T.  A key with st > T + 2 beta has s > T + beta, and
+//      every key that scores at least as much has st > T: it is among at most k-2 others, so it
+//      is selected whatever the ties do.  At least k keys have st >= T, hence s >= T - beta; a
+//      key with st < T - 2 beta has s < T - beta and is not selected.  The first kind gets +inf,
+//      the second -inf, the rest (a few hundred of 65536) are candidates.
+//   4. indexer_rescore_kernel: the reference's arithmetic, instruction for instruction as in
+//      indexer.hip, for the candidates only, spread over heads so that it takes microseconds.
+//   5. the exact top-k over the patched scores returns the reference's indices: the +inf keys
+//      are fewer than k and all belong to the selection, the -inf keys do not, and among the
+//      candidates the order is that of their exact scores and indices.
+// Whenever a row does not fit this (more candidates than the list holds, a bound that is not
+// finite, NaN where T should be), the exact kernel runs for that row after all: it is always
+// launched and returns at once for rows that went well.
+#include "common.hpp"
+
+namespace cwick {
+
+constexpr int IB_THREADS = 256;
+constexpr int IB_KEYS = 1024;                 // keys per workgroup of the approximate kernel
+constexpr int IB_HD = CWICK_HIP_INDEX_DIM;    // 128
+
+typedef __attribute__((ext_vector_type(2))) float ib_f32x2;
+
+__global__ void __launch_bounds__(IB_THREADS)
+indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict__ kscale,
+                      int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
+                      const uint16_t *__restrict__ q,   // [batch][ih][128] bf16
+                      const float *__restrict__ w,      // [batch][ih]
+                      int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
+                      IndexerBandRow *__restrict__ rows) {
+    __shared__ float c_sh[2][IB_HD];
+    __shared__ float w_sh[64];
+    __shared__ float bmax_sh[IB_THREADS / 64];
+    const int b = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint16_t *qb = q + (size_t)b * ih * IB_HD;
+    const float *wb = w + (size_t)b * ih;
+    if (wg == 0 && tid == 0) {
+        rows[b].n_cand = 0u;
+        rows[b].fallback = 0u;
+    }
+    // Contraction slot j of k-step ks in lane half g is dimension 64 g + 8 ks + j (the same on
+    // both operands, so the order is free): a lane reads 64 contiguous bytes of its key row,
+    // four 16-byte loads, and a wave reads 32 whole rows.
+    const int row = lane & 31, g = lane >> 5;
+    const uint8_t *kb = keys + (size_t)b * key_bstride;
+    const float *ksb = kscale + (size_t)b * kscale_bstride;
+    const int64_t wbase = (int64_t)wg * IB_KEYS + (int64_t)wave * (IB_KEYS / 4);
+    constexpr int N_IT = IB_KEYS / 4 / 32;
+    // the key bytes and the scale of an iteration are loaded two iterations ahead; the first
+    // two go out before anything else, so the cache streams while the operands are set up
+    u32x4 raw_a[4], raw_b[4];
+    float kst_a, kst_b;
+    auto load_keys = [&](int it, u32x4 (&raw)[4], float &kst) {
+        int64_t tc = wbase + (it < N_IT ? it : N_IT - 1) * 32 + row;
+        tc = tc < n_keys ? tc : n_keys - 1;
+        const uint8_t *krow = kb + (size_t)tc * IB_HD + 64 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) raw[i] = *(const u32x4 *)(krow + 16 * i);
+        kst = ksb[tc];
+    };
+    load_keys(0, raw_a, kst_a);
+    load_keys(1, raw_b, kst_b);
+
+    // A operands (rows = heads)
+    bf16x8 qa[2][8], ca[8];
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const int head = mb * 32 + row;
+            const int hc = head < ih ? head : ih - 1;           // clamped load, zeroed afterwards
+            u32x4 v = *(const u32x4 *)(qb + (size_t)hc * IB_HD + 64 * g + 8 * ks);
+            if (head >= ih) v = (u32x4){0u, 0u, 0u, 0u};
+            qa[mb][ks] = __builtin_bit_cast(bf16x8, v);
+        }
+    if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
+    {   // c_i = sum_h |w_h| |q_hi|: thread (i, half) takes 32 heads, all loads in flight at once
+        const int i = tid & (IB_HD - 1), half = tid >> 7;
+        uint16_t v[32];
+        float wa[32];
+#pragma unroll
+        for (int j = 0; j < 32; j++) {          // unconditional (clamped) loads: a guarded load is a branch
+            const int h = half * 32 + j;
+            const int hc = h < ih ? h : ih - 1;
+            v[j] = qb[(size_t)hc * IB_HD + i];
+            wa[j] = h < ih ? fabsf(wb[hc]) : 0.0f;
+        }
+        float c = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; j++) c += wa[j] * fabsf(bf16_to_f32(v[j]));
+        c_sh[half][i] = c;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row == 0) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                // rounded up to bf16
+                const int i0 = 64 * g + 8 * ks + 2 * j;
+                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0] + c_sh[1][i0]) + 0xFFFFu) >> 16;
+                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1] + c_sh[1][i0 + 1]) + 0xFFFFu) >> 16;
+                v[j] = lo | (hi << 16);
+            }
+        }
+        ca[ks] = __builtin_bit_cast(bf16x8, v);
+    }
+    // the heads this lane holds after the MFMAs: register i of block mb is head
+    // 32 mb + 8 (i / 4) + 4 g + i % 4
+    float wl[2][16];
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) wl[mb][i] = w_sh[mb * 32 + (i >> 2) * 8 + 4 * g + (i & 3)];
+
+    float bmax = 0.0f;
+    auto iteration = [&](int it, const u32x4 (&raw)[4], float kst) {
+        const int64_t t = wbase + it * 32 + row;
+        const bool live = t < n_keys;
+        // the accumulators are pinned to VGPRs (through the builtin they land in AGPRs and cost a
+        // read each); the compiler does not see these as MFMAs, hence the wait before the reads
+        f32x16 d0, d1, ab;
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            typedef __attribute__((ext_vector_type(2))) __bf16 ib_bf16x2;
+            u32x4 e;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {                          // exact: E4M3 fits bf16
+                const int dw = raw[ks >> 1][2 * (ks & 1) + j];
+                e[2 * j] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, false));
+                e[2 * j + 1] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, true));
+            }
+            u32x4 ea;
+#pragma unroll
+            for (int j = 0; j < 4; j++) ea[j] = e[j] & 0x7FFF7FFFu;
+            if (ks == 0) {
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d0) : "v"(qa[0][ks]), "v"(e));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d1) : "v"(qa[1][ks]), "v"(e));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(ab) : "v"(ca[ks]), "v"(ea));
+            } else {
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d0) : "v"(qa[0][ks]), "v"(e));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d1) : "v"(qa[1][ks]), "v"(e));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ab) : "v"(ca[ks]), "v"(ea));
+            }
+        }
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        float sp = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            sp = __builtin_fmaf(wl[0][i], __builtin_amdgcn_fmed3f(d0[i], 0.0f, INFINITY), sp);
+            sp = __builtin_fmaf(wl[1][i], __builtin_amdgcn_fmed3f(d1[i], 0.0f, INFINITY), sp);
+        }
+        sp += __shfl_xor(sp, 32, 64);
+        const float band = ab[0] + __shfl_xor(ab[0], 32, 64);      // row 0 sits in the g = 0 lanes
+        const float st = sp * kst;
+        const float beta = band * fabsf(kst) * (512.0f / 16777216.0f);
+        if (live && g == 0) scores[(size_t)b * n_keys + t] = st;
+        if (live) bmax = (beta <= bmax) ? bmax : beta;             // NaN sticks
+    };
+#pragma unroll 1
+    for (int it = 0; it < N_IT; it += 2) {
+        if (wbase + it * 32 >= n_keys) break;                      // wave-uniform
+        u32x4 raw[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) raw[i] = raw_a[i];
+        float kst = kst_a;
+        load_keys(it + 2, raw_a, kst_a);
+        iteration(it, raw, kst);
+        if (wbase + (it + 1) * 32 >= n_keys) break;
+#pragma unroll
+        for (int i = 0; i < 4; i++) raw[i] = raw_b[i];
+        kst = kst_b;
+        load_keys(it + 3, raw_b, kst_b);
+        iteration(it + 1, raw, kst);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float other = __shfl_xor(bmax, o, 64);
+        bmax = (other <= bmax) ? bmax : other;
+    }
+    if (lane == 0) bmax_sh[wave] = bmax;
+    __syncthreads();
+    if (tid == 0) {
+        float m = bmax_sh[0];
+#pragma unroll
+        for (int i = 1; i < IB_THREADS / 64; i++) m = (bmax_sh[i] <= m) ? m : bmax_sh[i];
+        beta_slots[(size_t)b * gridDim.x + wg] = m;
+    }
+}
+
+// The reference's score of each candidate, written over its approximate one.  One workgroup
+// = 16 candidates x 16 groups of four heads: lane j of a row of sixteen lanes holds candidate
+// j's key, the row its four heads; the dot products run exactly as in indexer_scores_kernel
+// (the q values of a head come to the FMAs through DPP row broadcasts); the 64 weighted terms
+// of a candidate meet in LDS and one lane adds them in head order.
+__global__ void __launch_bounds__(256)
+indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict__ kscale,
+                       int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
+                       const uint16_t *__restrict__ q, const float *__restrict__ w, int ih,
+                       const int32_t *__restrict__ cand, int cap,
+                       const IndexerBandRow *__restrict__ rows, float *__restrict__ scores) {
+    __shared__ float terms[16][65];
+    const int b = blockIdx.y, tid = threadIdx.x;
+    const IndexerBandRow st = rows[b];
+    if (indexer_band_failed(st, cap)) return;
+    const int c0 = blockIdx.x * 16;
+    if (c0 >= (int)st.n_cand) return;
+    const int j = tid & 15, hg = tid >> 4;                          // candidate, head group
+    const int ci = c0 + j < (int)st.n_cand ? c0 + j : (int)st.n_cand - 1;
+    const int64_t t = cand[(size_t)b * cap + ci];
+    const uint8_t *krow = keys + (size_t)b * key_bstride + (size_t)t * IB_HD;
+    const float ks = kscale[(size_t)b * kscale_bstride + t];
+    const uint16_t *qb = q + (size_t)b * ih * IB_HD;
+    const float *wb = w + (size_t)b * ih;
+    float e[IB_HD];
+#pragma unroll
+    for (int c = 0; c < IB_HD / 16; c++) {
+        const u32x4 v = *(const u32x4 *)(krow + c * 16);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const f32x2 lo = e4m3x2_to_f32<false>(v[jj]);
+            const f32x2 hi = e4m3x2_to_f32<true>(v[jj]);
+            e[c * 16 + jj * 4 + 0] = lo[0];
+            e[c * 16 + jj * 4 + 1] = lo[1];
+            e[c * 16 + jj * 4 + 2] = hi[0];
+            e[c * 16 + jj * 4 + 3] = hi[1];
+        }
+    }
+#pragma unroll 1
+    for (int hh = 0; hh < 4; hh++) {
+        const int h = hg * 4 + hh;
+        const int hc = h < ih ? h : ih - 1;
+        float qv[IB_HD / 16];                                       // lane j: q[h][16 c + j]
+#pragma unroll
+        for (int c = 0; c < IB_HD / 16; c++) qv[c] = bf16_to_f32(qb[(size_t)hc * IB_HD + 16 * c + j]);
+        // the loaded values pass through an (empty) VALU instruction: what the DPP reads below
+        // is then ordinary data to the compiler, which sees to the waits; the two wait states a
+        // DPP read needs after a VALU write are spent in the accumulator initialisation
+#pragma unroll
+        for (int c = 0; c < IB_HD / 16; c++) asm volatile("" : "+v"(qv[c]));
+        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+        asm volatile("s_nop 1" ::: "memory");
+#pragma unroll
+        for (int c = 0; c < IB_HD / 16; c++) {
+#define CWICK_IB_FMA(acc, n)                                                                       \
+    asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #n " row_mask:0xf bank_mask:0xf"       \
+                 : "+v"(acc) : "v"(qv[c]), "v"(e[16 * c + n]))
+            CWICK_IB_FMA(s0, 0);  CWICK_IB_FMA(s1, 1);  CWICK_IB_FMA(s2, 2);  CWICK_IB_FMA(s3, 3);
+            CWICK_IB_FMA(s0, 4);  CWICK_IB_FMA(s1, 5);  CWICK_IB_FMA(s2, 6);  CWICK_IB_FMA(s3, 7);
+            CWICK_IB_FMA(s0, 8);  CWICK_IB_FMA(s1, 9);  CWICK_IB_FMA(s2, 10); CWICK_IB_FMA(s3, 11);
+            CWICK_IB_FMA(s0, 12); CWICK_IB_FMA(s1, 13); CWICK_IB_FMA(s2, 14); CWICK_IB_FMA(s3, 15);
+#undef CWICK_IB_FMA
+        }
+        float d = (s0 + s1) + (s2 + s3);
+        d = d * ks;
+        d = d < 0.0f ? 0.0f : d;
+        const float prod = d * wb[hc];
+        terms[j][h] = h < ih ? prod : 0.0f;
+    }
+    __syncthreads();
+    if (tid < 16 && c0 + tid < (int)st.n_cand) {
+        float s = 0.0f;
+        for (int h = 0; h < ih; h++) s = s + terms[tid][h];
+        scores[(size_t)b * n_keys + cand[(size_t)b * cap + c0 + tid]] = s;
+    }
+}
+
+int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                          int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
+                          const float *w, int n_idx_heads, int64_t k, float *scores, hipStream_t s) {
+    CWICK_REQUIRE(keys && kscale && q_idx && w && scores, "indexer_banded: null pointer");
+    CWICK_REQUIRE(indexer_band_applies(n_keys, k, n_idx_heads), "indexer_banded: shape out of range");
+    CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
+                  "indexer_banded: keys and q must be 16-byte aligned");
+    const int n_wg = (int)((n_keys + IB_KEYS - 1) / IB_KEYS);
+    constexpr int cap = CWICK_INDEXER_BAND_CAP;
+    // workspace: [the top-k's slices and states][beta slots][row states][candidate lists]
+    const size_t topk_bytes = topk_mw_workspace_bytes(batch, n_keys);
+    size_t off_beta = (topk_bytes + 255) & ~(size_t)255;
+    size_t off_rows = off_beta + (((size_t)batch * n_wg * sizeof(float) + 255) & ~(size_t)255);
+    size_t off_cand = off_rows + (((size_t)batch * sizeof(IndexerBandRow) + 255) & ~(size_t)255);
+    const size_t total = off_cand + (size_t)batch * cap * sizeof(int32_t);
+    char *ws = (char *)workspace(s, total);
+    CWICK_REQUIRE(ws, "indexer_banded: workspace allocation failed");
+    float *beta_slots = (float *)(ws + off_beta);
+    IndexerBandRow *rows = (IndexerBandRow *)(ws + off_rows);
+    int32_t *cand = (int32_t *)(ws + off_cand);
+    ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
+    indexer_approx_kernel<<<dim3(n_wg, batch), IB_THREADS, 0, s>>>(
+        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows);
+    CWICK_HIP_CALL(hipGetLastError());
+    if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows, s))
+        return 0;
+    indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
+        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores);
+    CWICK_HIP_CALL(hipGetLastError());
+    // rows that did not fit the band take the exact kernel after all
+    return launch_indexer_scores_rows(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
+                                      n_idx_heads, scores, rows, cap, s);
+}
+
+}  // namespace cwick

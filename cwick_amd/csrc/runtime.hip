@@ -549,9 +549,21 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale, int64_t
     CWICK_REQUIRE(topk > 0 && n_keys > 0, "dsa_decode_dev: topk %lld n_keys %lld",
                   (long long)topk, (long long)n_keys);
     hipStream_t s = (hipStream_t)stream;
-    if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
-                               q_idx, w, n_idx_heads, scores_tmp, s))
+    // CWICK_HIP_INDEXER=exact scores every key with the exact kernel; the default scores most
+    // keys on the matrix cores and only the ones near the selection threshold exactly (the
+    // selected indices are the same)
+    static const bool exact_only = [] {
+        const char *e = getenv("CWICK_HIP_INDEXER");
+        return e && strcmp(e, "exact") == 0;
+    }();
+    if (!exact_only && indexer_band_applies(n_keys, topk, n_idx_heads)) {
+        if (!launch_indexer_banded(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
+                                   q_idx, w, n_idx_heads, topk, scores_tmp, s))
+            return 0;
+    } else if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch,
+                                      n_keys, q_idx, w, n_idx_heads, scores_tmp, s)) {
         return 0;
+    }
     if (!launch_topk(scores_tmp, batch, n_keys, topk, sel_out, s)) return 0;
     // rows past min(topk, n_keys) are -1 and are skipped by the attention kernel
     return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_keys, batch,

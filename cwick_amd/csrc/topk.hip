@@ -523,6 +523,90 @@ topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
     }
 }
 
+// The select half of the banded indexer (indexer_band.hip): T is the k-th largest approximate
+// score, beta the largest error bound of the row; scores above T + 2 beta become +inf, scores
+// below T - 2 beta become -inf, the rest stay and are listed for exact rescoring.
+__global__ void __launch_bounds__(TOPK_MW_THREADS)
+topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
+                        const uint32_t *__restrict__ ws, size_t ws_row,
+                        const float *__restrict__ beta_slots, int n_beta,
+                        int32_t *__restrict__ cand, int cap, IndexerBandRow *__restrict__ rows) {
+    __shared__ uint32_t hist[256];
+    __shared__ TopkMwState sh_state;
+    __shared__ float sh_beta[TOPK_MW_THREADS / 64];
+    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const uint32_t *slices = ws + (size_t)row * ws_row;
+    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    float *sc = scores + (size_t)row * n;
+    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
+    float v[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        v[j] = i < n ? sc[i] : 0.0f;
+    }
+    float beta = tid < n_beta ? beta_slots[(size_t)row * n_beta + tid] : 0.0f;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float other = __shfl_xor(beta, o, 64);
+        beta = (other <= beta) ? beta : other;                  // NaN sticks
+    }
+    if (lane == 0) sh_beta[tid >> 6] = beta;
+    // three digits are enough here: the k-th largest key lies in the bucket [T_lo, T_hi] of the
+    // 24-bit prefix; at most k-1 keys lie above the bucket and at least k in or above it, which
+    // is all the argument needs, and the bucket is 256 ulps wide, far inside beta
+    const TopkMwState st = topk_mw_pick(slices + (size_t)2 * n_wg * 256, n_wg, 8, state[2], hist, &sh_state);
+    beta = sh_beta[0];
+#pragma unroll
+    for (int i = 1; i < TOPK_MW_THREADS / 64; i++) beta = (sh_beta[i] <= beta) ? beta : sh_beta[i];
+    // the floats behind the order keys
+    auto key_float = [](uint32_t key) -> float {
+        return __builtin_bit_cast(float, (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
+    };
+    const float T_lo = key_float(st.prefix), T_hi = key_float(st.prefix | 0xFFu);
+    const bool ok = (st.prefix >> 8) != 0u && beta >= 0.0f && beta < INFINITY && T_lo == T_lo && T_hi == T_hi;
+    if (!ok) {
+        if (wg == 0 && tid == 0) rows[row].fallback = 1u;
+        return;
+    }
+    const float hi = T_hi + 2.004f * beta, lo = T_lo - 2.004f * beta;
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        if (i < n) {
+            if (v[j] > hi) sc[i] = INFINITY;
+            else if (v[j] < lo) sc[i] = -INFINITY;
+            else {
+                const uint32_t slot = atomicAdd(&rows[row].n_cand, 1u);
+                if (slot < (uint32_t)cap) cand[(size_t)row * cap + slot] = (int32_t)i;
+            }
+        }
+    }
+}
+
+static size_t topk_mw_row_dwords(int64_t n_wg) { return (size_t)4 * n_wg * 256 + 2 * 4; }
+
+size_t topk_mw_workspace_bytes(int batch, int64_t n) {
+    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
+    return (size_t)batch * topk_mw_row_dwords(n_wg) * sizeof(uint32_t);
+}
+
+int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
+                              const float *beta_slots, int n_beta, int32_t *cand, int cap,
+                              IndexerBandRow *rows, hipStream_t s) {
+    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
+    CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && n_beta <= TOPK_MW_THREADS,
+                  "topk_band_classify: n %lld out of range", (long long)n);
+    const size_t ws_row = topk_mw_row_dwords(n_wg);
+    const dim3 grid((unsigned)n_wg, (unsigned)batch);
+    for (int pass = 0; pass < 3; pass++)
+        topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row);
+    topk_mw_classify_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, beta_slots,
+                                                            n_beta, cand, cap, rows);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s) {
     CWICK_REQUIRE(scores && out_idx, "topk: null pointer");
@@ -531,7 +615,7 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
     const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
     if (n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS) {
-        const size_t ws_row = (size_t)4 * n_wg * 256 + 2 * 4;       // dwords: slices, then four states
+        const size_t ws_row = topk_mw_row_dwords(n_wg);             // dwords: slices, then four states
         uint32_t *ws = (uint32_t *)workspace(s, (size_t)batch * ws_row * sizeof(uint32_t));
         CWICK_REQUIRE(ws, "topk: workspace allocation failed");
         const dim3 grid((unsigned)n_wg, (unsigned)batch);

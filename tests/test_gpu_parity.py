@@ -265,8 +265,9 @@ def test_topk_bit_exact(hip, orc, n, k, kind):
 
 
 @pytest.mark.parametrize("n_keys,topk", [
-    (3000, 256),         # one workgroup per query in the top-k
-    (20000, 512),        # many workgroups per query, batched
+    (3000, 256),         # every key scored exactly; one workgroup per query in the top-k
+    (20000, 512),        # approximate scores + exact band, many workgroups per query, batched
+    (65536, 2048),       # BASELINE config 5 geometry (batch 3)
 ])
 def test_dsa_decode_small(hip, orc, n_keys, topk):
     say("[case] dsa_decode small", n_keys, topk)
@@ -283,5 +284,35 @@ def test_dsa_decode_small(hip, orc, n_keys, topk):
         assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
         ref = orc.mla_decode(c["q"][b], c["rows"][b], c["scales"][b], c["scale"], sel=rsel, nthreads=0)
         assert_close(out[b], ref, "dsa_decode query %d" % b)
+    ik.free()
+    lat.free()
+
+
+@pytest.mark.parametrize("kind", ["same", "two", "zero_w"])
+def test_dsa_select_degenerate(hip, orc, kind):
+    """Selections where the error band of the approximate scores holds most keys (identical or
+    nearly identical scores): the exact kernel has to take over, the indices stay the
+    reference's (lowest index first among ties)."""
+    say("[case] dsa select degenerate", kind)
+    n_keys, topk = 20000, 512
+    c = synth.cfg5_dsa(n_keys=n_keys, batch=2, ih=64, topk=topk, nh=128, seed=911)
+    ikeys = c["ikeys"].copy(); ikscale = c["ikscale"].copy(); w = c["w"].copy()
+    if kind == "same":
+        ikeys[:] = ikeys[:, :1]; ikscale[:] = ikscale[:, :1]          # every key the same
+    elif kind == "two":
+        ikeys[:, 1::2] = ikeys[:, :1]; ikscale[:, 1::2] = ikscale[:, :1]
+        ikeys[:, 0::2] = ikeys[:, 1:2]; ikscale[:, 0::2] = ikscale[:, 1:2]
+    else:
+        w[:] = 0.0                                                     # all scores zero
+    ik = hip.IndexKeys(2, n_keys)
+    lat = hip.LatentCache(2, n_keys)
+    for b in range(2):
+        ik.write(b, 0, ikeys[b], ikscale[b])
+        lat.write(b, 0, c["rows"][b], c["scales"][b])
+    out, sel = hip.dsa_decode(ik, lat, 0, 1, n_keys, c["q_idx"], w, topk, c["q"], c["scale"])
+    for b in range(2):
+        sc = orc.indexer_scores(c["q_idx"][b], w[b], ikeys[b], ikscale[b], nthreads=0)
+        rsel = orc.topk_contract(sc, topk)
+        assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
     ik.free()
     lat.free()
