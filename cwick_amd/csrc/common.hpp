@@ -71,6 +71,14 @@ struct IndexerBandRow {
     uint32_t fallback;    // the band could not be formed (bound not finite, NaN threshold)
 };
 constexpr int CWICK_INDEXER_BAND_CAP = 4096;   // candidate list entries per row
+constexpr int CWICK_INDEXER_APPROX_KEYS = 1024;   // keys per workgroup (= per bound slot) of the approximate kernel
+inline int indexer_approx_slots(int64_t n_keys) {
+    return (int)((n_keys + CWICK_INDEXER_APPROX_KEYS - 1) / CWICK_INDEXER_APPROX_KEYS);
+}
+int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                          int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
+                          const float *w, int n_idx_heads, float *scores, float *beta_slots,
+                          IndexerBandRow *rows, hipStream_t s);
 __host__ __device__ inline bool indexer_band_failed(const IndexerBandRow &r, int cap) {
     return r.fallback != 0u || r.n_cand > (uint32_t)cap;
 }

@@ -37,7 +37,7 @@
 namespace cwick {
 
 constexpr int IB_THREADS = 256;
-constexpr int IB_KEYS = 1024;                 // keys per workgroup of the approximate kernel
+constexpr int IB_KEYS = CWICK_INDEXER_APPROX_KEYS;   // keys per workgroup of the approximate kernel
 constexpr int IB_HD = CWICK_HIP_INDEX_DIM;    // 128
 
 typedef __attribute__((ext_vector_type(2))) float ib_f32x2;
@@ -288,6 +288,23 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
     }
 }
 
+// the approximate scores and the per-workgroup maxima of their error bound (the first stage of
+// the banded select on its own; n_keys / IB_KEYS slots per row, rounded up)
+int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_bstride,
+                          int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
+                          const float *w, int n_idx_heads, float *scores, float *beta_slots,
+                          IndexerBandRow *rows, hipStream_t s) {
+    CWICK_REQUIRE(keys && kscale && q_idx && w && scores && beta_slots && rows, "indexer_approx: null pointer");
+    CWICK_REQUIRE(n_keys >= 1 && n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_approx: shape out of range");
+    CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
+                  "indexer_approx: keys and q must be 16-byte aligned");
+    const int n_wg = indexer_approx_slots(n_keys);
+    indexer_approx_kernel<<<dim3(n_wg, batch), IB_THREADS, 0, s>>>(
+        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
 int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
                           const float *w, int n_idx_heads, int64_t k, float *scores, hipStream_t s) {
@@ -295,7 +312,7 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     CWICK_REQUIRE(indexer_band_applies(n_keys, k, n_idx_heads), "indexer_banded: shape out of range");
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
                   "indexer_banded: keys and q must be 16-byte aligned");
-    const int n_wg = (int)((n_keys + IB_KEYS - 1) / IB_KEYS);
+    const int n_wg = indexer_approx_slots(n_keys);
     constexpr int cap = CWICK_INDEXER_BAND_CAP;
     // workspace: [the top-k's slices and states][beta slots][row states][candidate lists]
     const size_t topk_bytes = topk_mw_workspace_bytes(batch, n_keys);
@@ -309,9 +326,9 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     IndexerBandRow *rows = (IndexerBandRow *)(ws + off_rows);
     int32_t *cand = (int32_t *)(ws + off_cand);
     ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
-    indexer_approx_kernel<<<dim3(n_wg, batch), IB_THREADS, 0, s>>>(
-        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows);
-    CWICK_HIP_CALL(hipGetLastError());
+    if (!launch_indexer_approx(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w, n_idx_heads,
+                               scores, beta_slots, rows, s))
+        return 0;
     if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows, s))
         return 0;
     indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(

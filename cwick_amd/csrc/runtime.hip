@@ -707,6 +707,41 @@ int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys, const
     return 1;
 }
 
+int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys,
+                                    const uint16_t *q_idx, const float *w, int n_idx_heads,
+                                    float *scores, float *bound) {
+    clear_error();
+    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    CWICK_REQUIRE(c && q_idx && w && scores && bound, "indexer_scores_approx: null argument");
+    CWICK_REQUIRE(slot >= 0 && slot < c->slots, "indexer_scores_approx: slot %d of %d", slot, c->slots);
+    CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "indexer_scores_approx: n_keys %lld, capacity %lld",
+                  (long long)n_keys, (long long)c->capacity);
+    CWICK_REQUIRE(n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_scores_approx: n_idx_heads %d (1..64)",
+                  n_idx_heads);
+    const int n_slots = indexer_approx_slots(n_keys);
+    size_t qb = (size_t)n_idx_heads * CWICK_HIP_INDEX_DIM * 2, wb = (size_t)n_idx_heads * 4;
+    size_t ob = (size_t)n_keys * 4, bb = (size_t)n_slots * 4;
+    char *st = (char *)staging(nullptr, pad256(qb) + pad256(wb) + pad256(ob) + pad256(bb) + 256);
+    CWICK_REQUIRE(st, "indexer_scores_approx: staging allocation failed");
+    size_t off = 0;
+    uint16_t *dq = (uint16_t *)stage_in(st, off, q_idx, qb);
+    float *dw = (float *)stage_in(st, off, w, wb);
+    CWICK_REQUIRE(dq && dw, "indexer_scores_approx: upload failed");
+    float *dout = (float *)(st + off);
+    float *dbeta = (float *)(st + off + pad256(ob));
+    IndexerBandRow *drow = (IndexerBandRow *)(st + off + pad256(ob) + pad256(bb));
+    if (!launch_indexer_approx(cwick_hip_ikeys_rows_dev(c, slot), cwick_hip_ikeys_scales_dev(c, slot), 0, 0,
+                               1, n_keys, dq, dw, n_idx_heads, dout, dbeta, drow, nullptr))
+        return 0;
+    CWICK_HIP_CALL(hipMemcpy(scores, dout, ob, hipMemcpyDeviceToHost));
+    std::vector<float> hb((size_t)n_slots);
+    CWICK_HIP_CALL(hipMemcpy(hb.data(), dbeta, bb, hipMemcpyDeviceToHost));
+    float m = hb[0];
+    for (int i = 1; i < n_slots; i++) m = (hb[i] <= m) ? m : hb[i];      // NaN sticks
+    *bound = m;
+    return 1;
+}
+
 int cwick_hip_topk(const float *scores, int64_t n, int64_t k, int32_t *out_idx, int64_t *n_out) {
     clear_error();
     CWICK_REQUIRE(backend_ready(), "backend not ready");
@@ -800,7 +835,7 @@ int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches) {
 const char *cwick_hip_prof_name(int which) {
     static const char *names[CWICK_HIP_PROF_COUNT] = {
         "gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk kernels"};
+        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels"};
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 

@@ -58,6 +58,7 @@ SIGNATURES = {
     "cwick_hip_mla_decode": (_int, [_vp, _int, _vp, _i64, _vp, _int, _flt, _vp]),
     "cwick_hip_mla_prefill_chunk": (_int, [_vp, _int, _i64, _i64, _vp, _int, _flt, _vp]),
     "cwick_hip_indexer_scores": (_int, [_vp, _int, _i64, _vp, _vp, _int, _vp]),
+    "cwick_hip_indexer_scores_approx": (_int, [_vp, _int, _i64, _vp, _vp, _int, _vp, C.POINTER(_flt)]),
     "cwick_hip_topk": (_int, [_vp, _i64, _i64, _vp, C.POINTER(_i64)]),
     "cwick_hip_dsa_decode": (_int, [_vp, _vp, _int, _int, _int, _i64, _vp, _vp, _int, _i64,
                                     _vp, _int, _flt, _vp, _vp]),
@@ -317,6 +318,17 @@ def indexer_scores(ikeys, slot, n_keys, q_idx, w, raw=False):
     return out
 
 
+def indexer_scores_approx(ikeys, slot, n_keys, q_idx, w):
+    """(approximate scores, bound): |approximate - exact| <= bound for every key of the row."""
+    q, qp = _np(q_idx, np.uint16)
+    w, wp = _np(w, np.float32)
+    out = np.empty(n_keys, np.float32)
+    bound = _flt(0.0)
+    _check(lib().cwick_hip_indexer_scores_approx(ikeys.h, slot, n_keys, qp, wp, q.shape[0],
+                                                 out.ctypes.data, C.byref(bound)), "indexer_scores_approx")
+    return out, float(bound.value)
+
+
 def topk(scores, k, raw=False):
     s, sp = _np(scores, np.float32)
     out = np.empty(max(k, 1), np.int32)
@@ -404,7 +416,7 @@ def dsa_decode_dev(ikeys, ikscale, key_bstride, kscale_bstride, rows, scales, ro
 
 # ------------------------------------------------------------------ phase timers
 PROF_NAMES = ["gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer_scores_kernel", "topk kernels"]
+              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels"]
 
 
 def prof_enable(on=True):

@@ -174,6 +174,16 @@ int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys,
                              const uint16_t *q_idx, const float *w, int n_idx_heads,
                              float *scores);
 
+/* No counterpart in the reference: the first stage of the fused select
+ * (cwick_hip_dsa_decode), on its own, for checking it.  scores[t] approximates
+ * the score above on the matrix cores; *bound is one number for the row with
+ * |scores[t] - exact score[t]| <= *bound for every t (see indexer_band.hip for
+ * the derivation).  The fused call scores exactly only the keys whose
+ * approximate score lies within 2 * bound of the selection threshold. */
+int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys,
+                                    const uint16_t *q_idx, const float *w, int n_idx_heads,
+                                    float *scores, float *bound);
+
 /* Replaces ds_topk_scores (src/ds_ops.c:310-338, contract src/ds_ops.h:110-112)
  * and the threshold selector of src/attention.c:585-598: the k best of n
  * scores by (score descending, index ascending), written in ascending index
@@ -255,7 +265,7 @@ enum {
     CWICK_HIP_PROF_GQA_PREFILL,         /* gqa_prefill_kernel */
     CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill) */
     CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag16_kernel after it */
-    CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel */
+    CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel, or in a fused select indexer_approx_kernel + 3 x topk_mw_hist_kernel + topk_mw_classify_kernel + indexer_rescore_kernel + the exact kernel's fallback pass */
     CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel */
     CWICK_HIP_PROF_COUNT
 };

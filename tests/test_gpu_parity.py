@@ -219,6 +219,38 @@ def test_indexer_scores_bit_exact(hip, orc, n_keys, ih):
     cache.free()
 
 
+@pytest.mark.parametrize("n_keys,ih,kind", [
+    (65536, 64, "normal"), (20000, 64, "positive_w"), (5000, 7, "normal"), (40000, 33, "wide"),
+])
+def test_indexer_approx_within_its_bound(hip, orc, n_keys, ih, kind):
+    """The matrix-core scores of the fused select and the bound that comes with them: every key's
+    approximate score must lie within the bound of the exact one (the selection relies on it),
+    and the bound must be small against the spread of the scores (or the band holds everything).
+    Measured against the oracle's exact scores, which the exact kernel reproduces bit for bit."""
+    say("[case] indexer approx bound", n_keys, ih, kind)
+    g = synth.rng(520 + n_keys + ih)
+    keys, ks = synth.index_keys(g, n_keys)
+    q = synth.normal_bf16(g, (ih, synth.IDIM))
+    w = (g.standard_normal(ih, dtype=np.float32) / np.float32(np.sqrt(128.0 * ih))).astype(np.float32)
+    if kind == "positive_w":
+        w = np.abs(w)
+    if kind == "wide":                              # scales and queries over many binades
+        ks = (ks * np.exp2(g.integers(-20, 20, n_keys)).astype(np.float32)).astype(np.float32)
+        q = synth.f32_to_bf16(synth.bf16_to_f32(q) * np.exp2(g.integers(-8, 8, (ih, 1))).astype(np.float32))
+    cache = hip.IndexKeys(1, n_keys)
+    cache.write(0, 0, keys, ks)
+    approx, bound = hip.indexer_scores_approx(cache, 0, n_keys, q, w)
+    ref = orc.indexer_scores(q, w, keys, ks, nthreads=0)
+    err = np.abs(approx.astype(np.float64) - ref.astype(np.float64))
+    say("[bound] max error %.3e, bound %.3e (error/bound %.3f), score std %.3e" %
+        (err.max(), bound, err.max() / bound, ref.std()))
+    assert np.isfinite(bound) and bound > 0
+    assert err.max() <= bound, "approximate scores leave their bound: %.3e > %.3e" % (err.max(), bound)
+    if kind != "wide":
+        assert bound < 1e-2 * ref.std(), "the bound is useless: %.3e against a spread of %.3e" % (bound, ref.std())
+    cache.free()
+
+
 TOPK_KNOWN = [
     ([5, 5, 7], 2, [0, 2]),                      # ds_topk_scores returns {1,2} here
     ([3, 9, 3, 3, 8, 3], 4, [0, 1, 2, 4]),       # ... and {1,2,3,4} here
