@@ -49,7 +49,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       const float *__restrict__ w,      // [batch][ih]
                       int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
                       IndexerBandRow *__restrict__ rows) {
-    __shared__ float c_sh[2][IB_HD];
+    __shared__ float c_sh[1][IB_HD];
     __shared__ float w_sh[64];
     __shared__ float bmax_sh[IB_THREADS / 64];
     const int b = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
@@ -68,8 +68,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     const float *ksb = kscale + (size_t)b * kscale_bstride;
     const int64_t wbase = (int64_t)wg * IB_KEYS + (int64_t)wave * (IB_KEYS / 4);
     constexpr int N_IT = IB_KEYS / 4 / 32;
-    // the key bytes and the scale of an iteration are loaded two iterations ahead; the first
-    // two go out before anything else, so the cache streams while the operands are set up
+    // the key bytes and the scale of an iteration are loaded two iterations ahead
     u32x4 raw_a[4], raw_b[4];
     float kst_a, kst_b;
     auto load_keys = [&](int it, u32x4 (&raw)[4], float &kst) {
@@ -80,10 +79,9 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         for (int i = 0; i < 4; i++) raw[i] = *(const u32x4 *)(krow + 16 * i);
         kst = ksb[tc];
     };
-    load_keys(0, raw_a, kst_a);
-    load_keys(1, raw_b, kst_b);
-
-    // A operands (rows = heads)
+    // A operands (rows = heads).  Their loads go out first and the first two key iterations
+    // right behind them: loads return in order, so the bound row below is worked out of the
+    // operand registers while the keys are still on their way
     bf16x8 qa[2][8], ca[8];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
@@ -96,21 +94,39 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
             qa[mb][ks] = __builtin_bit_cast(bf16x8, v);
         }
     if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
-    {   // c_i = sum_h |w_h| |q_hi|: thread (i, half) takes 32 heads, all loads in flight at once
-        const int i = tid & (IB_HD - 1), half = tid >> 7;
-        uint16_t v[32];
-        float wa[32];
+    const float w0_abs = row < ih ? fabsf(wb[row]) : 0.0f;
+    const float w1_abs = row + 32 < ih ? fabsf(wb[row + 32]) : 0.0f;
+    load_keys(0, raw_a, kst_a);
+    load_keys(1, raw_b, kst_b);
+    {   // c_i = sum_h |w_h| |q_hi| from the operand registers: lane (row, g) holds dims 64 g .. +63
+        // of heads row and row + 32; a reduce-scatter over the 32 lanes of a half (exchange half
+        // of the values, add, five times) leaves dims 64 g + 2 row + {0, 1} in each lane
+        const float w0 = w0_abs, w1 = w1_abs;
+        float val[64];
 #pragma unroll
-        for (int j = 0; j < 32; j++) {          // unconditional (clamped) loads: a guarded load is a branch
-            const int h = half * 32 + j;
-            const int hc = h < ih ? h : ih - 1;
-            v[j] = qb[(size_t)hc * IB_HD + i];
-            wa[j] = h < ih ? fabsf(wb[hc]) : 0.0f;
+        for (int ks = 0; ks < 8; ks++) {
+            const u32x4 x0 = __builtin_bit_cast(u32x4, qa[0][ks]), x1 = __builtin_bit_cast(u32x4, qa[1][ks]);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                val[8 * ks + 2 * j] = w0 * fabsf(bf16lo_to_f32(x0[j])) + w1 * fabsf(bf16lo_to_f32(x1[j]));
+                val[8 * ks + 2 * j + 1] = w0 * fabsf(bf16hi_to_f32(x0[j])) + w1 * fabsf(bf16hi_to_f32(x1[j]));
+            }
         }
-        float c = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 32; j++) c += wa[j] * fabsf(bf16_to_f32(v[j]));
-        c_sh[half][i] = c;
+#define CWICK_IB_RS(m, n)                                                                \
+    {                                                                                    \
+        const bool up = (lane & (m)) != 0;                                               \
+        _Pragma("unroll") for (int i = 0; i < (n); i++) {                                \
+            const float send = up ? val[i] : val[i + (n)];                               \
+            const float keep = up ? val[i + (n)] : val[i];                               \
+            val[i] = keep + __shfl_xor(send, (m), 64);                                   \
+        }                                                                                \
+    }
+        CWICK_IB_RS(16, 32) CWICK_IB_RS(8, 16) CWICK_IB_RS(4, 8) CWICK_IB_RS(2, 4) CWICK_IB_RS(1, 2)
+#undef CWICK_IB_RS
+        if (wave == 0) {
+            c_sh[0][64 * g + 2 * row] = val[0];
+            c_sh[0][64 * g + 2 * row + 1] = val[1];
+        }
     }
     __syncthreads();
 #pragma unroll
@@ -121,8 +137,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
             for (int j = 0; j < 4; j++) {
                 // rounded up to bf16
                 const int i0 = 64 * g + 8 * ks + 2 * j;
-                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0] + c_sh[1][i0]) + 0xFFFFu) >> 16;
-                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1] + c_sh[1][i0 + 1]) + 0xFFFFu) >> 16;
+                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0]) + 0xFFFFu) >> 16;
+                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1]) + 0xFFFFu) >> 16;
                 v[j] = lo | (hi << 16);
             }
         }
@@ -249,13 +265,22 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
             e[c * 16 + jj * 4 + 3] = hi[1];
         }
     }
-#pragma unroll 1
+    // q of the group's four heads, all loads in flight at once: lane j holds q[h][16 c + j]
+    float qall[4][IB_HD / 16], wh[4];
+#pragma unroll
     for (int hh = 0; hh < 4; hh++) {
         const int h = hg * 4 + hh;
         const int hc = h < ih ? h : ih - 1;
-        float qv[IB_HD / 16];                                       // lane j: q[h][16 c + j]
 #pragma unroll
-        for (int c = 0; c < IB_HD / 16; c++) qv[c] = bf16_to_f32(qb[(size_t)hc * IB_HD + 16 * c + j]);
+        for (int c = 0; c < IB_HD / 16; c++) qall[hh][c] = bf16_to_f32(qb[(size_t)hc * IB_HD + 16 * c + j]);
+        wh[hh] = wb[hc];
+    }
+#pragma unroll
+    for (int hh = 0; hh < 4; hh++) {
+        const int h = hg * 4 + hh;
+        float qv[IB_HD / 16];
+#pragma unroll
+        for (int c = 0; c < IB_HD / 16; c++) qv[c] = qall[hh][c];
         // the loaded values pass through an (empty) VALU instruction: what the DPP reads below
         // is then ordinary data to the compiler, which sees to the waits; the two wait states a
         // DPP read needs after a VALU write are spent in the accumulator initialisation
@@ -277,7 +302,7 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
         float d = (s0 + s1) + (s2 + s3);
         d = d * ks;
         d = d < 0.0f ? 0.0f : d;
-        const float prod = d * wb[hc];
+        const float prod = d * wh[hh];
         terms[j][h] = h < ih ? prod : 0.0f;
     }
     __syncthreads();
