@@ -311,16 +311,19 @@ constexpr int TOPK_MW_MAX_WGS = 64;                              // per row
 
 struct TopkMwState { uint32_t prefix, remaining; };
 
-// sum of p[w * 256] over w < count with sixteen loads in flight (the slices sit in L2: a
-// dependent chain of loads would cost a round trip each)
+// sum of p[w * 256] over w < count with thirty-two loads in flight (the slices sit in L2: a
+// dependent chain of loads would cost a round trip each, and so does every further batch)
 __device__ __forceinline__ uint32_t topk_mw_colsum(const uint32_t *__restrict__ p, int count) {
     uint32_t c = 0u;
-    for (int w0 = 0; w0 < count; w0 += 16) {
-        uint32_t v[16];
+    for (int w0 = 0; w0 < count; w0 += 32) {
+        uint32_t v[32];
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = w0 + j < count ? p[(size_t)(w0 + j) * 256] : 0u;
+        for (int j = 0; j < 32; j++) {
+            const int w = w0 + j < count ? w0 + j : count - 1;      // clamped, not guarded: a guarded load is a branch
+            v[j] = p[(size_t)w * 256];
+        }
 #pragma unroll
-        for (int j = 0; j < 16; j++) c += v[j];
+        for (int j = 0; j < 32; j++) c += w0 + j < count ? v[j] : 0u;
     }
     return c;
 }
@@ -386,8 +389,24 @@ topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
     TopkMwState st{0u, (uint32_t)kk};
     if (pass > 0) {
         if (pass > 1) st = state[pass - 1];
+        // this workgroup's own bin of the previous pass: issued before the pick, used after it
+        const uint32_t own_prev = slices[((size_t)(pass - 1) * n_wg + wg) * 256 + tid];
         st = topk_mw_pick(slices + (size_t)(pass - 1) * n_wg * 256, n_wg, 32 - 8 * pass, st, hist, &sh_state);
         if (wg == 0 && tid == 0) state[pass] = st;
+        // how many of this workgroup's keys left the chosen path at the previous digit with a
+        // larger bin, i.e. lie above T whatever the later digits are: the emit kernel adds
+        // these up over the workgroups before it
+        const uint32_t dig = (st.prefix >> (32 - 8 * pass)) & 0xFFu;
+        uint32_t above = (uint32_t)tid > dig ? own_prev : 0u;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) above += __shfl_xor(above, o, 64);
+        if ((tid & 63) == 0) hist8[tid >> 6] = above;
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t *abv = (uint32_t *)(state + 4);
+            abv[(size_t)(pass - 1) * n_wg + wg] = hist8[0] + hist8[1] + hist8[2] + hist8[3];
+        }
+        __syncthreads();
     }
     const int shift = 24 - 8 * pass;
     const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (32 - 8 * pass));
@@ -434,28 +453,15 @@ topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
         const int64_t i = base + j * TOPK_MW_THREADS + tid;
         keys[j] = i < n ? topk_key(sc[i]) : 0u;
     }
-    // keys above T in the workgroups before this one, part 1: bin `tid` of pass p of workgroup w
-    // counts keys that match the chosen digits 0..p-1 and have digit p = tid; they are above T
-    // if tid is larger than the chosen digit p.  Digits 0..2 are known before the last pick:
-    // their loads go out together and travel while it runs.
+    // keys above T in the workgroups before this one, part 1: bin b of pass p of workgroup w
+    // counts keys that match the chosen digits 0..p-1 and have digit p = b; they are above T if
+    // b is larger than the chosen digit p
     const TopkMwState st3 = state[3];
     uint32_t gt = 0u, eq = 0u;
-    {
-        bool above[3];
-#pragma unroll
-        for (int p = 0; p < 3; p++) above[p] = (uint32_t)tid > ((st3.prefix >> (24 - 8 * p)) & 0xFFu);
-        for (int w0 = 0; w0 < wg; w0 += 8) {
-            uint32_t v[3][8];
-#pragma unroll
-            for (int p = 0; p < 3; p++)
-#pragma unroll
-                for (int j = 0; j < 8; j++)
-                    v[p][j] = (above[p] && w0 + j < wg) ? slices[((size_t)p * n_wg + w0 + j) * 256 + tid] : 0u;
-#pragma unroll
-            for (int p = 0; p < 3; p++)
-#pragma unroll
-                for (int j = 0; j < 8; j++) gt += v[p][j];
-        }
+    {   // digits 0..2: the histogram kernels left one count per workgroup and digit
+        const uint32_t *abv = (const uint32_t *)(state + 4);
+        const int p = tid / TOPK_MW_MAX_WGS, w = tid % TOPK_MW_MAX_WGS;     // 3 x 64 <= 256 threads
+        if (p < 3 && w < wg) gt = abv[(size_t)p * n_wg + w];
     }
     const TopkMwState st = topk_mw_pick(slices + (size_t)3 * n_wg * 256, n_wg, 0, st3, hist, &sh_state);
     const uint32_t T = st.prefix, r = st.remaining;   // r ties belong to the selection
@@ -584,7 +590,9 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     }
 }
 
-static size_t topk_mw_row_dwords(int64_t n_wg) { return (size_t)4 * n_wg * 256 + 2 * 4; }
+// a row's workspace in dwords: slices[4][n_wg][256], four states, above[3][n_wg] (+ padding to
+// keep the rows 8-byte aligned)
+static size_t topk_mw_row_dwords(int64_t n_wg) { return (size_t)4 * n_wg * 256 + 2 * 4 + (size_t)((3 * n_wg + 1) & ~(int64_t)1); }
 
 size_t topk_mw_workspace_bytes(int batch, int64_t n) {
     const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
