@@ -16,8 +16,8 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libcwick_hip.so")
 
-SOURCES = ["runtime.hip", "misc.hip", "gqa_decode.hip", "gqa_prefill.hip", "mla.hip",
-           "mla_stream.hip", "mla_dsplit.hip", "mla_roles.hip", "indexer.hip", "indexer_band.hip", "topk.hip"]
+SOURCES = ["runtime.hip", "misc.hip", "gqa_decode.hip", "gqa_prefill.hip", "mla_roles.hip",
+           "indexer.hip", "indexer_band.hip", "topk.hip"]
 
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
           "-Wall", "-Wno-unused-function",

@@ -1,7 +1,5 @@
 // mla_roles.hip -- absorbed-latent MLA over the FP8 latent (decode, sparse decode and chunked
-// prefill of src/attention.c:749-811 / :1010-1019).  This is the kernel the entry points use;
-// mla_dsplit.hip, mla_stream.hip and mla.hip are earlier schedules kept selectable
-// (CWICK_HIP_MLA=dsplit|stream|v1) as comparison arms.
+// prefill of src/attention.c:749-811 / :1010-1019).
 //
 //   workgroup = 12 waves, 32 query rows (heads of one query) x one key slice, walked in tiles
 //   of 64 keys.  The waves take one of two roles:
@@ -45,25 +43,6 @@
 #include <cstring>
 
 namespace cwick {
-int launch_mla_decode_v1(const uint8_t *rows, const float *scales, int64_t row_bstride,
-                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                         hipStream_t s);
-int launch_mla_prefill_v1(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
-                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
-int launch_mla_decode_v2(const uint8_t *rows, const float *scales, int64_t row_bstride,
-                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                         hipStream_t s);
-int launch_mla_prefill_v2(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
-                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
-int launch_mla_decode_v3(const uint8_t *rows, const float *scales, int64_t row_bstride,
-                         int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                         int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                         hipStream_t s);
-int launch_mla_prefill_v3(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
-                          const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
-
 namespace {
 
 constexpr int KDIM = CWICK_HIP_LATENT_KDIM;   // 576
@@ -712,16 +691,6 @@ int run(Params &p, hipStream_t s) {
     return 1;
 }
 
-// CWICK_HIP_MLA = v1 | stream | dsplit selects an earlier schedule (comparison arms)
-int variant() {
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("CWICK_HIP_MLA");
-        v = !e ? 0 : (!strcmp(e, "v1") ? 1 : (!strcmp(e, "stream") ? 2 : (!strcmp(e, "dsplit") ? 3 : 0)));
-    }
-    return v;
-}
-
 int splits_per_cu() {
     static int v = -1;
     if (v < 0) {
@@ -738,15 +707,6 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
                       int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
                       hipStream_t s) {
-    if (variant() == 1)
-        return launch_mla_decode_v1(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
-                                    q, n_heads, scale, out, s);
-    if (variant() == 2)
-        return launch_mla_decode_v2(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
-                                    q, n_heads, scale, out, s);
-    if (variant() == 3)
-        return launch_mla_decode_v3(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list,
-                                    q, n_heads, scale, out, s);
     CWICK_REQUIRE(rows && scales && q && out, "mla_decode: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 4096, "mla_decode: batch %d", batch);
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
@@ -778,9 +738,6 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
 
 int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
                        const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s) {
-    if (variant() == 1) return launch_mla_prefill_v1(rows, scales, pos0, n, q, n_heads, scale, out, s);
-    if (variant() == 2) return launch_mla_prefill_v2(rows, scales, pos0, n, q, n_heads, scale, out, s);
-    if (variant() == 3) return launch_mla_prefill_v3(rows, scales, pos0, n, q, n_heads, scale, out, s);
     CWICK_REQUIRE(rows && scales && q && out, "mla_prefill: null pointer");
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill: n_heads %d (1..128)", n_heads);
     CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= ((int64_t)1 << 31) - 1 && n <= (1 << 22),
