@@ -296,14 +296,15 @@ def test_topk_bit_exact(hip, orc, n, k, kind):
     assert np.array_equal(got, ref)
 
 
-@pytest.mark.parametrize("n_keys,topk", [
-    (3000, 256),         # every key scored exactly; one workgroup per query in the top-k
-    (20000, 512),        # approximate scores + exact band, many workgroups per query, batched
-    (65536, 2048),       # BASELINE config 5 geometry (batch 3)
+@pytest.mark.parametrize("n_keys,topk,ih", [
+    (3000, 256, 64),     # every key scored exactly; one workgroup per query in the top-k
+    (20000, 512, 64),    # approximate scores + exact band, many workgroups per query, batched
+    (65536, 2048, 64),   # BASELINE config 5 geometry (batch 3)
+    (17000, 300, 22),    # fewer index heads than the kernels' blocks of 32 and groups of 4
 ])
-def test_dsa_decode_small(hip, orc, n_keys, topk):
-    say("[case] dsa_decode small", n_keys, topk)
-    c = synth.cfg5_dsa(n_keys=n_keys, batch=3, ih=64, topk=topk, nh=128, seed=909)
+def test_dsa_decode_small(hip, orc, n_keys, topk, ih):
+    say("[case] dsa_decode small", n_keys, topk, ih)
+    c = synth.cfg5_dsa(n_keys=n_keys, batch=3, ih=ih, topk=topk, nh=128, seed=909)
     ik = hip.IndexKeys(3, n_keys)
     lat = hip.LatentCache(3, n_keys)
     for b in range(3):
