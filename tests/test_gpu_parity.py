@@ -77,6 +77,7 @@ def test_gqa_decode(hip, orc, n_keys, nh, nkv, hd):
     (1990, 200, 4, 4),       # group 1
     (1000, 100, 8, 4),       # the boundary between the variants inside a chunk
     (3000, 40, 16, 2),       # group 8, a chunk shorter than one position block
+    (1500, 260, 4, 2),       # group 2, two position blocks and a ragged third
 ])
 def test_gqa_prefill(hip, orc, pos0, n, nh, nkv):
     say("[case] gqa_prefill", pos0, n, nh, nkv)
