@@ -184,7 +184,9 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
             }
         }
         const int h = g * GROUP + j;
-        part_acc[((size_t)split * n_heads + h) * HD + d] = a;
+        // written through: the merge kernel reads it from other XCDs, and a dirty line would be
+        // written back at the end of this kernel
+        __hip_atomic_store(&part_acc[((size_t)split * n_heads + h) * HD + d], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (d == 0) {
             part_ml[((size_t)split * n_heads + h) * 2 + 0] = mx;
             part_ml[((size_t)split * n_heads + h) * 2 + 1] = ls;

@@ -64,6 +64,8 @@ constexpr int MERGE_MAX_SPLITS = 1024;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+// the larger of two values; a NaN on either side wins
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a || a > b) ? a : b; }
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -81,7 +83,8 @@ struct Params {
     float scale;
     int n_splits;
     int64_t keys_per_split;   // multiple of TK
-    float *out, *part_acc, *part_ml;
+    float *out, *part_ml;
+    uint32_t *part_acc;
 };
 
 struct Tile {
@@ -548,106 +551,151 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             const float unit_f = e_run == E_NONE ? 0.0f : pow2i(e_run - WEXP);   // the accumulators are in units of 2^(e_run - WEXP)
             const float fin = p.n_splits == 1 ? (L > 0.0f ? unit_f / L : 0.0f) : unit_f;
             const size_t pb = ((size_t)y * p.n_splits + split) * (2 * n_hb) + 2 * hb + h2;
+            if (p.n_splits == 1) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    // accumulator register i <-> dim 16 db + 4 g + i
+                    const f32x4 v = oacc[h2][j] * fin;
+                    *(f32x4 *)(p.out + ((size_t)y * p.nh + head) * VDIM + 16 * (8 * cw + j) + 4 * g) = v;
+                }
+                continue;
+            }
+            // The partial leaves as 16-bit fixed point: this wave's 128 dims of the head share one
+            // scale, their largest magnitude, so every value is off by at most 2^-16 of that.  A
+            // non-finite value makes the scale NaN and with it the head's merged output.
+            float big = 0.0f;   // in accumulator units
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) big = nan_max(big, __builtin_fabsf(oacc[h2][j][i]));
+            big = nan_max(big, __shfl_xor(big, 16));
+            big = nan_max(big, __shfl_xor(big, 32));
+            if (!(big < INFINITY)) big = __builtin_nanf("");
+            const float to_unit = big > 0.0f ? 1.0f / big : 0.0f;
+            uint32_t *pq = p.part_acc + (pb * NDB + 8 * cw) * 128 + lane * 2;   // [db][lane][4 x i16]
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const int db = 8 * cw + j;
-                const f32x4 v = oacc[h2][j] * fin;
-                // accumulator register i <-> dim 16 db + 4 g + i
-                if (p.n_splits == 1) *(f32x4 *)(p.out + ((size_t)y * p.nh + head) * VDIM + 16 * db + 4 * g) = v;
-                else *(f32x4 *)(p.part_acc + pb * (HB * VDIM) + ((size_t)db * 64 + lane) * 4) = v;   // [db][lane][4]
+                const f32x4 v = oacc[h2][j] * to_unit;
+                u32x2 w;
+                w[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(v[0], v[1]));
+                w[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(v[2], v[3]));
+                // written through to memory as it is stored: the merge runs on other XCDs, and what
+                // would otherwise sit dirty in this L2 is written back at the end of the kernel,
+                // on the critical path (about 1 us for the 8 MB of a full-chip launch)
+                __hip_atomic_store((uint64_t *)(pq + j * 128), __builtin_bit_cast(uint64_t, w), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
             }
-            if (p.n_splits > 1 && cw == 0 && g == 0) {
-                p.part_ml[(pb * HB + n) * 2 + 0] = m_ref[h2] * 0.69314718055994530942f;
-                p.part_ml[(pb * HB + n) * 2 + 1] = L;
-            }
+            if (g == 0)
+                *(f32x4 *)(p.part_ml + ((pb * 4 + cw) * HB + n) * 4) =
+                    (f32x4){m_ref[h2] * 0.69314718055994530942f, L, big * fin * (1.0f / 32767.0f), 0.0f};
         }
     }
 }
 
-// merge of fragment-layout partials [y][split][16-head block][dim block][lane][4]: workgroup =
-// one dim block of one 16-head block; its waves (up to sixteen, one per split when there are
-// fewer) take splits w, w + n_waves, ... and meet in LDS.  Every wave has all its loads in
-// flight at once (eight splits per batch); which splits exist is uniform per wave, so absent
-// ones cost nothing.
+// merge of fragment-layout partials: values [y][split][16-head block][dim block][lane][4] as
+// 16-bit fixed point, and per 16-head block and quarter of the dims [head][4] floats (running
+// maximum in natural-log units, weight sum, value of one fixed-point step, unused).  With more
+// than eight splits a workgroup is one dim block of one 16-head block: its sixteen waves take
+// splits w, w + 16, ... and meet in LDS.  With up to eight a wave merges a dim block alone and
+// eight of them make a workgroup (a batch of queries splits each query less: one wave per
+// split would be thousands of workgroups that each wait out one load).  Every wave has all its
+// loads in flight at once (eight splits per batch); which splits exist is uniform per wave, so
+// absent ones cost nothing.
 constexpr int MW = 16;
+__device__ __forceinline__ void merge_add(f32x4 &acc, float &ls, const u32x2 a, const f32x4 v, const float mx) {
+    const float c = v[0] == -INFINITY ? 0.0f : __expf(v[0] - mx);
+    ls = __builtin_fmaf(v[1], c, ls);
+    const float cs = c * v[2];
+    acc[0] = __builtin_fmaf((float)((int32_t)(a[0] << 16) >> 16), cs, acc[0]);
+    acc[1] = __builtin_fmaf((float)((int32_t)a[0] >> 16), cs, acc[1]);
+    acc[2] = __builtin_fmaf((float)((int32_t)(a[1] << 16) >> 16), cs, acc[2]);
+    acc[3] = __builtin_fmaf((float)((int32_t)a[1] >> 16), cs, acc[3]);
+}
 __global__ void __launch_bounds__(64 * MW)
-mla_merge_frag16_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
-                        int n_splits, int n_hb16, int nh, float *__restrict__ out) {
+mla_merge_frag16_kernel(const uint32_t *__restrict__ part_acc, const float *__restrict__ part_ml,
+                        int n_splits, int n_hb16, int nh, float *__restrict__ out, int packed) {
     __shared__ float red_m[MW][64];
     __shared__ float red_l[MW][64];
     __shared__ f32x4 red_a[MW][64];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), mw = (int)blockDim.x >> 6;
-    const int db = blockIdx.x % NDB, hb = blockIdx.x / NDB, y = blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), y = blockIdx.y;
+    int wv, mw, db, hb;
+    if (packed) {
+        // up to eight splits: a wave merges a dim block by itself, and the workgroup's eight
+        // waves take the eight dim blocks of one quarter
+        wv = 0, mw = 1, db = 8 * (int)(blockIdx.x & 3) + wave, hb = (int)(blockIdx.x >> 2);
+    } else {
+        // workgroups go to the eight XCDs round robin: the eight dim blocks that share a quarter's
+        // [head][4] floats sit on one XCD, so that only one L2 fetches them (n_hb16 is even)
+        const int grp = (int)(blockIdx.x & 7) + 8 * (int)(blockIdx.x >> 6);
+        wv = wave, mw = (int)blockDim.x >> 6;
+        db = 8 * (grp & 3) + (int)((blockIdx.x >> 3) & 7), hb = grp >> 2;
+    }
     const int n = lane & 15, g = lane >> 4;
     const size_t sb = (size_t)y * n_splits;
-    const float *ml = part_ml + ((sb * n_hb16 + hb) * HB + n) * 2;
-    const size_t ml_stride = (size_t)n_hb16 * HB * 2;
-    const float *pa = part_acc + (sb * n_hb16 + hb) * (HB * VDIM) + ((size_t)db * 64 + lane) * 4;
-    const size_t pa_stride = (size_t)n_hb16 * HB * VDIM;
+    const float *ml = part_ml + (((sb * n_hb16 + hb) * 4 + (db >> 3)) * HB + n) * 4;
+    const size_t ml_stride = (size_t)n_hb16 * 4 * HB * 4;
+    const uint32_t *pa = part_acc + ((sb * n_hb16 + hb) * NDB + db) * 128 + lane * 2;
+    const size_t pa_stride = (size_t)n_hb16 * NDB * 128;
 
     // first batch: everything in flight before anything is waited for
-    f32x4 a0[8];
-    f32x2 v0[8];
+    u32x2 a0[8];
+    f32x4 v0[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const int s = wv + mw * j;
-        v0[j] = (f32x2){-INFINITY, 0.0f};
-        a0[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        v0[j] = (f32x4){-INFINITY, 0.0f, 0.0f, 0.0f};
+        a0[j] = (u32x2){0u, 0u};
         if (s < n_splits) {
-            v0[j] = *(const f32x2 *)(ml + s * ml_stride);
-            a0[j] = *(const f32x4 *)(pa + s * pa_stride);
+            v0[j] = *(const f32x4 *)(ml + s * ml_stride);
+            a0[j] = *(const u32x2 *)(pa + s * pa_stride);
         }
     }
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; j++) mx = fmaxf(mx, v0[j][0]);
     for (int s = wv + 8 * mw; s < n_splits; s += mw) mx = fmaxf(mx, ml[s * ml_stride]);
-    red_m[wv][lane] = mx;
-    __syncthreads();
-    for (int w = 0; w < mw; w++) mx = fmaxf(mx, red_m[w][lane]);
+    if (mw > 1) {
+        red_m[wv][lane] = mx;
+        __syncthreads();
+        for (int w = 0; w < mw; w++) mx = fmaxf(mx, red_m[w][lane]);
+    }
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float ls = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float c = v0[j][0] == -INFINITY ? 0.0f : __expf(v0[j][0] - mx);
-        ls = __builtin_fmaf(v0[j][1], c, ls);
-#pragma unroll
-        for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(a0[j][r], c, acc[r]);
-    }
+    for (int j = 0; j < 8; j++) merge_add(acc, ls, a0[j], v0[j], mx);
     for (int s0 = wv + 8 * mw; s0 < n_splits; s0 += 8 * mw) {
-        f32x4 a[8];
-        f32x2 v[8];
+        u32x2 a[8];
+        f32x4 v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int s = s0 + mw * j;
-            v[j] = (f32x2){-INFINITY, 0.0f};
-            a[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            v[j] = (f32x4){-INFINITY, 0.0f, 0.0f, 0.0f};
+            a[j] = (u32x2){0u, 0u};
             if (s < n_splits) {
-                v[j] = *(const f32x2 *)(ml + s * ml_stride);
-                a[j] = *(const f32x4 *)(pa + s * pa_stride);
+                v[j] = *(const f32x4 *)(ml + s * ml_stride);
+                a[j] = *(const u32x2 *)(pa + s * pa_stride);
             }
         }
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float c = v[j][0] == -INFINITY ? 0.0f : __expf(v[j][0] - mx);
-            ls = __builtin_fmaf(v[j][1], c, ls);
-#pragma unroll
-            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(a[j][r], c, acc[r]);
-        }
+        for (int j = 0; j < 8; j++) merge_add(acc, ls, a[j], v[j], mx);
     }
-    red_l[wv][lane] = ls;
-    red_a[wv][lane] = acc;
-    __syncthreads();
-    if (wv != 0) return;
-    float l = 0.f;
-    f32x4 r4 = {0.f, 0.f, 0.f, 0.f};
-    for (int w = 0; w < mw; w++) {
-        l += red_l[w][lane];
-        const f32x4 t = red_a[w][lane];
+    float l = ls;
+    f32x4 r4 = acc;
+    if (mw > 1) {
+        red_l[wv][lane] = ls;
+        red_a[wv][lane] = acc;
+        __syncthreads();
+        if (wv != 0) return;
+        l = 0.f;
+        r4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int w = 0; w < mw; w++) {
+            l += red_l[w][lane];
+            const f32x4 t = red_a[w][lane];
 #pragma unroll
-        for (int r = 0; r < 4; r++) r4[r] += t[r];
+            for (int r = 0; r < 4; r++) r4[r] += t[r];
+        }
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const int head = hb * HB + n;
@@ -670,11 +718,11 @@ int run(Params &p, hipStream_t s) {
     const int64_t total = (int64_t)n_hb * p.n_splits * p.nq;
     CWICK_REQUIRE(total <= 0x7FFFFFFF, "mla: grid of %lld workgroups is too large", (long long)total);
     if (p.n_splits > 1) {
-        const size_t acc_b = (size_t)p.nq * p.n_splits * n_hb * HW * VDIM * sizeof(float);
-        const size_t ml_b = (size_t)p.nq * p.n_splits * n_hb * HW * 2 * sizeof(float);
+        const size_t acc_b = (size_t)p.nq * p.n_splits * n_hb * HW * VDIM * sizeof(int16_t);
+        const size_t ml_b = (size_t)p.nq * p.n_splits * n_hb * HW * 4 * 4 * sizeof(float);
         char *ws = (char *)workspace(s, acc_b + ml_b);
         CWICK_REQUIRE(ws, "mla: workspace allocation failed");
-        p.part_acc = (float *)ws;
+        p.part_acc = (uint32_t *)ws;
         p.part_ml = (float *)(ws + acc_b);
     }
     {
@@ -684,8 +732,12 @@ int run(Params &p, hipStream_t s) {
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
         ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
-        mla_merge_frag16_kernel<<<dim3(2 * n_hb * NDB, p.nq), 64 * (p.n_splits < MW ? p.n_splits : MW), 0, s>>>(
-            p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out);
+        if (p.n_splits <= 8)
+            mla_merge_frag16_kernel<<<dim3(2 * n_hb * 4, p.nq), 64 * 8, 0, s>>>(
+                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out, 1);
+        else
+            mla_merge_frag16_kernel<<<dim3(2 * n_hb * NDB, p.nq), 64 * MW, 0, s>>>(
+                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out, 0);
         CWICK_HIP_CALL(hipGetLastError());
     }
     return 1;
