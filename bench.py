@@ -131,8 +131,8 @@ def bench_cfg3(hip, synth, T, stream):
     t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
     # HBM bytes of one launch of mla_roles_kernel at this geometry (64 key slices): FETCH_SIZE and
     # WRITE_SIZE of rocprofv3 --pmc, each scaled by what a 256 MiB copy reads on the same counter
-    # (profiles/mla_decode_cfg3_pmc_traffic.txt): 20.97 MB read + 16.84 MB of split-K partials written
-    traffic = 20482 * 1024 + 16448 * 1024
+    # (profiles/mla_decode_cfg3_pmc_traffic.txt): 21.00 MB read + 8.91 MB of split-K partials written
+    traffic = 20512 * 1024 + 8704 * 1024
     return {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
                         "+ 5 fp32 block scales/token, bf16 q",
             "us_per_step": wall * 1e6, "kernels": kern, "alg_bytes": alg, "flops": flops,

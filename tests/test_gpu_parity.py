@@ -167,6 +167,33 @@ def test_mla_decode_dense(hip, orc, n_keys, nh):
     cache.free()
 
 
+@pytest.mark.parametrize("n_keys,gain", [(4096, 32.0), (32768, 32.0), (3000, 8.0)])
+def test_mla_decode_large_values(hip, orc, n_keys, gain):
+    """Latent values `gain` times larger with the query's latent part as much smaller: the same
+    scores, outputs `gain` times larger.  The split partials cross HBM as 16-bit fixed point with
+    one scale per head and 128 dims, good to 2^-16 of the largest of those outputs, so the
+    elementwise tolerance holds while that largest output stays below about a hundred.  The
+    second value block is made another 16 times smaller: small outputs next to no large one."""
+    say("[case] mla_decode large values", n_keys, gain)
+    c = synth.cfg3_mla_decode(n_keys, 128, seed=900 + n_keys)
+    scales = c["scales"].copy()
+    scales[:, :4] *= np.float32(gain)
+    scales[:, 1] *= np.float32(1.0 / 16.0)
+    qf = synth.bf16_to_f32(c["q"]).copy()
+    qf[:, :512] *= np.float32(1.0 / gain)                  # powers of two: exact in bf16
+    qf[:, 128:256] *= np.float32(16.0)
+    q = synth.f32_to_bf16(qf)
+    cache = hip.LatentCache(1, n_keys)
+    cache.write(0, 0, c["rows"], scales)
+    got = hip.mla_decode(cache, 0, q, c["scale"], n_list=n_keys)
+    ref = orc.mla_decode(q, c["rows"], scales, c["scale"], nthreads=0)
+    assert np.abs(ref).max() < 100.0
+    assert_close(got, ref, "mla_decode values x%g, %d keys" % (gain, n_keys), strict=False)
+    blk = np.abs(got[:, 128:256] - ref[:, 128:256]).max()
+    say("[parity] small block: max-abs %.3e of max |ref| %.3e" % (blk, np.abs(ref[:, 128:256]).max()))
+    cache.free()
+
+
 def test_mla_decode_sel(hip, orc):
     say("[case] mla_decode sel")
     n_rows, nh = 5000, 128
