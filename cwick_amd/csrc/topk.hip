@@ -576,17 +576,36 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
         return;
     }
     const float hi = T_hi + 2.004f * beta, lo = T_lo - 2.004f * beta;
+    // candidates take a place in the workgroup first (LDS counter), the workgroup then takes its
+    // run of the row's list with one atomic: a few hundred returning atomics on one address from
+    // all over the chip would queue up behind each other
+    uint32_t *wg_count = &hist[0], *wg_base = &hist[1];          // the pick is done with hist
+    if (tid == 0) *wg_count = 0u;
+    __syncthreads();
+    uint32_t is_cand = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_MW_EPT; j++) {
         const int64_t i = base + j * TOPK_MW_THREADS + tid;
         if (i < n) {
             if (v[j] > hi) sc[i] = INFINITY;
             else if (v[j] < lo) sc[i] = -INFINITY;
-            else {
-                const uint32_t slot = atomicAdd(&rows[row].n_cand, 1u);
-                if (slot < (uint32_t)cap) cand[(size_t)row * cap + slot] = (int32_t)i;
-            }
+            else is_cand |= 1u << j;
         }
+    }
+    uint32_t my_first = 0u;
+    const uint32_t mine = (uint32_t)__builtin_popcount(is_cand);
+    if (mine) my_first = atomicAdd(wg_count, mine);
+    __syncthreads();
+    if (tid == 0) *wg_base = *wg_count ? atomicAdd(&rows[row].n_cand, *wg_count) : 0u;
+    __syncthreads();
+    if (mine) {
+        uint32_t slot = *wg_base + my_first;
+#pragma unroll
+        for (int j = 0; j < TOPK_MW_EPT; j++)
+            if (is_cand >> j & 1u) {
+                if (slot < (uint32_t)cap) cand[(size_t)row * cap + slot] = (int32_t)(base + j * TOPK_MW_THREADS + tid);
+                slot++;
+            }
     }
 }
 
