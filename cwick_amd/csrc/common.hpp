@@ -78,7 +78,8 @@ inline int indexer_approx_slots(int64_t n_keys) {
 int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
                           const float *w, int n_idx_heads, float *scores, float *beta_slots,
-                          IndexerBandRow *rows, hipStream_t s);
+                          IndexerBandRow *rows, uint32_t *digit0_slices, size_t digit0_row_dwords,
+                          hipStream_t s);
 __host__ __device__ inline bool indexer_band_failed(const IndexerBandRow &r, int cap) {
     return r.fallback != 0u || r.n_cand > (uint32_t)cap;
 }
@@ -96,10 +97,14 @@ int launch_indexer_scores_rows(const uint8_t *keys, const float *kscale, int64_t
                                const IndexerBandRow *rows, int cap, hipStream_t s);
 // top-k machinery on approximate scores: finds T, then patches the scores (+inf / -inf / kept)
 // and lists the keys within 2 beta of T.  `ws` holds topk_mw_workspace_bytes() at its start.
+// With `digit0_done` the first-digit counts are already there: the approximate kernel left one
+// 256-bin slice per workgroup (indexer_approx_slots(n) of them) at the start of each row's
+// workspace, rows topk_mw_band_row_dwords(n) dwords apart.
 size_t topk_mw_workspace_bytes(int batch, int64_t n);
+size_t topk_mw_band_row_dwords(int64_t n);
 int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
                               const float *beta_slots, int n_beta, int32_t *cand, int cap,
-                              IndexerBandRow *rows, hipStream_t s);
+                              IndexerBandRow *rows, bool digit0_done, hipStream_t s);
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s);
 int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,
@@ -110,6 +115,15 @@ int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
 
 // ---- device helpers ---------------------------------------------------------
+// order-preserving 32-bit key of a score for the radix select: larger score, larger key; NaN
+// sorts below everything (key 0), -0.0 equals +0.0, and no number maps to 0
+__device__ __forceinline__ uint32_t topk_key(float f) {
+    if (f != f) return 0u;
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u << 1) == 0u) u = 0u;                       // -0.0 -> +0.0
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return u == 0u ? 1u : u;
+}
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;

@@ -48,8 +48,10 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       const uint16_t *__restrict__ q,   // [batch][ih][128] bf16
                       const float *__restrict__ w,      // [batch][ih]
                       int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
-                      IndexerBandRow *__restrict__ rows) {
+                      IndexerBandRow *__restrict__ rows,
+                      uint32_t *__restrict__ digit0, size_t digit0_row) {   // optional: first-digit counts for the radix select
     __shared__ float c_sh[1][IB_HD];
+    __shared__ uint32_t hist0[256 * 8];
     __shared__ float w_sh[64];
     __shared__ float bmax_sh[IB_THREADS / 64];
     const int b = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
@@ -94,6 +96,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
             qa[mb][ks] = __builtin_bit_cast(bf16x8, v);
         }
     if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) hist0[tid + IB_THREADS * j] = 0u;
     const float w0_abs = row < ih ? fabsf(wb[row]) : 0.0f;
     const float w1_abs = row + 32 < ih ? fabsf(wb[row + 32]) : 0.0f;
     load_keys(0, raw_a, kst_a);
@@ -193,7 +197,12 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         const float band = ab[0] + __shfl_xor(ab[0], 32, 64);      // row 0 sits in the g = 0 lanes
         const float st = sp * kst;
         const float beta = band * fabsf(kst) * (512.0f / 16777216.0f);
-        if (live && g == 0) scores[(size_t)b * n_keys + t] = st;
+        if (live && g == 0) {
+            scores[(size_t)b * n_keys + t] = st;
+            // the select's first pass over the scores, done here: the leading byte of the order
+            // key, counted in eight copies picked by lane (scores crowd into a few bins)
+            atomicAdd(&hist0[(topk_key(st) >> 24) * 8 + (lane & 7)], 1u);
+        }
         if (live) bmax = (beta <= bmax) ? bmax : beta;             // NaN sticks
     };
 #pragma unroll 1
@@ -224,6 +233,12 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
 #pragma unroll
         for (int i = 1; i < IB_THREADS / 64; i++) m = (bmax_sh[i] <= m) ? m : bmax_sh[i];
         beta_slots[(size_t)b * gridDim.x + wg] = m;
+    }
+    if (digit0) {
+        uint32_t c = 0u;
+#pragma unroll
+        for (int j = 0; j < 8; j++) c += hist0[tid * 8 + ((j + tid) & 7)];
+        digit0[(size_t)b * digit0_row + (size_t)wg * 256 + tid] = c;
     }
 }
 
@@ -318,14 +333,17 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
 int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
                           const float *w, int n_idx_heads, float *scores, float *beta_slots,
-                          IndexerBandRow *rows, hipStream_t s) {
+                          IndexerBandRow *rows, uint32_t *digit0_slices, size_t digit0_row_dwords,
+                          hipStream_t s) {
+    static_assert(IB_THREADS == 256, "one thread per first-digit bin");
     CWICK_REQUIRE(keys && kscale && q_idx && w && scores && beta_slots && rows, "indexer_approx: null pointer");
     CWICK_REQUIRE(n_keys >= 1 && n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_approx: shape out of range");
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
                   "indexer_approx: keys and q must be 16-byte aligned");
     const int n_wg = indexer_approx_slots(n_keys);
     indexer_approx_kernel<<<dim3(n_wg, batch), IB_THREADS, 0, s>>>(
-        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows);
+        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows,
+        digit0_slices, digit0_row_dwords);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }
@@ -352,9 +370,10 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     int32_t *cand = (int32_t *)(ws + off_cand);
     ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
     if (!launch_indexer_approx(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w, n_idx_heads,
-                               scores, beta_slots, rows, s))
+                               scores, beta_slots, rows, (uint32_t *)ws, topk_mw_band_row_dwords(n_keys), s))
         return 0;
-    if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows, s))
+    if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows,
+                                   true, s))
         return 0;
     indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
         keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores);

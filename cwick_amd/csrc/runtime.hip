@@ -731,7 +731,7 @@ int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys
     float *dbeta = (float *)(st + off + pad256(ob));
     IndexerBandRow *drow = (IndexerBandRow *)(st + off + pad256(ob) + pad256(bb));
     if (!launch_indexer_approx(cwick_hip_ikeys_rows_dev(c, slot), cwick_hip_ikeys_scales_dev(c, slot), 0, 0,
-                               1, n_keys, dq, dw, n_idx_heads, dout, dbeta, drow, nullptr))
+                               1, n_keys, dq, dw, n_idx_heads, dout, dbeta, drow, nullptr, 0, nullptr))
         return 0;
     CWICK_HIP_CALL(hipMemcpy(scores, dout, ob, hipMemcpyDeviceToHost));
     std::vector<float> hb((size_t)n_slots);

@@ -30,14 +30,6 @@ namespace cwick {
 constexpr int TOPK_THREADS = 1024;
 constexpr int TOPK_WAVES = TOPK_THREADS / 64;
 
-__device__ __forceinline__ uint32_t topk_key(float f) {
-    if (f != f) return 0u;
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u << 1) == 0u) u = 0u;                       // -0.0 -> +0.0
-    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-    return u == 0u ? 1u : u;
-}
-
 // exclusive scan of one value per thread across the block; returns the
 // exclusive prefix and writes the block total to *total
 __device__ __forceinline__ uint32_t block_exscan(uint32_t v, uint32_t *sh_wave, uint32_t *total) {
@@ -366,16 +358,19 @@ topk_mw_pick(const uint32_t *__restrict__ slices, int n_wg, int shift, TopkMwSta
     return out;
 }
 
-// workspace of a row: slices[4][n_wg][256], then state[4]
+// workspace of a row: slices[4][sl][256], then state[4], then above[3][n_wg].  sl >= n_wg slices
+// are laid out per pass; passes 1..3 use n_wg of them, pass 0 uses n_s0: its counts may come
+// from another kernel that cut the row into more pieces (each an equal share of a workgroup's
+// keys here).
 __global__ void __launch_bounds__(TOPK_MW_THREADS)
 topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int n_wg, int pass,
-                    uint32_t *__restrict__ ws, size_t ws_row) {
+                    uint32_t *__restrict__ ws, size_t ws_row, int sl, int n_s0) {
     __shared__ uint32_t hist[256];
     __shared__ uint32_t hist8[256 * 8];
     __shared__ TopkMwState sh_state;
     const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x;
     uint32_t *slices = ws + (size_t)row * ws_row;
-    TopkMwState *state = (TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    TopkMwState *state = (TopkMwState *)(slices + (size_t)4 * sl * 256);
     const int64_t kk = k < n ? k : n;
     // the workgroup's scores: issued first, they travel while the previous digit is picked
     const float *sc = scores + (size_t)row * n;
@@ -390,8 +385,16 @@ topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
     if (pass > 0) {
         if (pass > 1) st = state[pass - 1];
         // this workgroup's own bin of the previous pass: issued before the pick, used after it
-        const uint32_t own_prev = slices[((size_t)(pass - 1) * n_wg + wg) * 256 + tid];
-        st = topk_mw_pick(slices + (size_t)(pass - 1) * n_wg * 256, n_wg, 32 - 8 * pass, st, hist, &sh_state);
+        uint32_t own_prev;
+        if (pass == 1) {
+            const int per = (n_s0 + n_wg - 1) / n_wg;             // pass-0 slices per workgroup
+            own_prev = 0u;
+            for (int j = 0; j < per; j++)
+                if (wg * per + j < n_s0) own_prev += slices[((size_t)wg * per + j) * 256 + tid];
+        } else {
+            own_prev = slices[((size_t)(pass - 1) * sl + wg) * 256 + tid];
+        }
+        st = topk_mw_pick(slices + (size_t)(pass - 1) * sl * 256, pass == 1 ? n_s0 : n_wg, 32 - 8 * pass, st, hist, &sh_state);
         if (wg == 0 && tid == 0) state[pass] = st;
         // how many of this workgroup's keys left the chosen path at the previous digit with a
         // larger bin, i.e. lie above T whatever the later digits are: the emit kernel adds
@@ -427,12 +430,12 @@ topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
     uint32_t c = 0u;
 #pragma unroll
     for (int j = 0; j < 8; j++) c += hist8[tid * 8 + ((j + tid) & 7)];
-    slices[((size_t)pass * n_wg + wg) * 256 + tid] = c;
+    slices[((size_t)pass * sl + wg) * 256 + tid] = c;
 }
 
 __global__ void __launch_bounds__(TOPK_MW_THREADS)
 topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
-                    const uint32_t *__restrict__ ws, size_t ws_row, int32_t *__restrict__ out) {
+                    const uint32_t *__restrict__ ws, size_t ws_row, int sl, int32_t *__restrict__ out) {
     __shared__ uint32_t hist[256];
     __shared__ TopkMwState sh_state;
     __shared__ uint32_t sh_red[2][TOPK_MW_THREADS / 64];
@@ -440,7 +443,7 @@ topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
     const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t *slices = ws + (size_t)row * ws_row;
-    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * sl * 256);
     int32_t *dst = out + (size_t)row * k;
     const int64_t kk = k < n ? k : n;
     if (wg == 0)
@@ -463,12 +466,12 @@ topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
         const int p = tid / TOPK_MW_MAX_WGS, w = tid % TOPK_MW_MAX_WGS;     // 3 x 64 <= 256 threads
         if (p < 3 && w < wg) gt = abv[(size_t)p * n_wg + w];
     }
-    const TopkMwState st = topk_mw_pick(slices + (size_t)3 * n_wg * 256, n_wg, 0, st3, hist, &sh_state);
+    const TopkMwState st = topk_mw_pick(slices + (size_t)3 * sl * 256, n_wg, 0, st3, hist, &sh_state);
     const uint32_t T = st.prefix, r = st.remaining;   // r ties belong to the selection
     {   // part 2: the last digit; equal to T if it is the digit itself
         const uint32_t dig = T & 0xFFu;
         const bool above = (uint32_t)tid > dig, same = (uint32_t)tid == dig;
-        const uint32_t c = topk_mw_colsum(slices + (size_t)3 * n_wg * 256 + tid, (above || same) ? wg : 0);
+        const uint32_t c = topk_mw_colsum(slices + (size_t)3 * sl * 256 + tid, (above || same) ? wg : 0);
         if (above) gt += c;
         if (same) eq += c;
     }
@@ -536,13 +539,13 @@ __global__ void __launch_bounds__(TOPK_MW_THREADS)
 topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
                         const uint32_t *__restrict__ ws, size_t ws_row,
                         const float *__restrict__ beta_slots, int n_beta,
-                        int32_t *__restrict__ cand, int cap, IndexerBandRow *__restrict__ rows) {
+                        int32_t *__restrict__ cand, int cap, IndexerBandRow *__restrict__ rows, int sl) {
     __shared__ uint32_t hist[256];
     __shared__ TopkMwState sh_state;
     __shared__ float sh_beta[TOPK_MW_THREADS / 64];
     const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const uint32_t *slices = ws + (size_t)row * ws_row;
-    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * n_wg * 256);
+    const TopkMwState *state = (const TopkMwState *)(slices + (size_t)4 * sl * 256);
     float *sc = scores + (size_t)row * n;
     const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
     float v[TOPK_MW_EPT];
@@ -561,7 +564,7 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     // three digits are enough here: the k-th largest key lies in the bucket [T_lo, T_hi] of the
     // 24-bit prefix; at most k-1 keys lie above the bucket and at least k in or above it, which
     // is all the argument needs, and the bucket is 256 ulps wide, far inside beta
-    const TopkMwState st = topk_mw_pick(slices + (size_t)2 * n_wg * 256, n_wg, 8, state[2], hist, &sh_state);
+    const TopkMwState st = topk_mw_pick(slices + (size_t)2 * sl * 256, n_wg, 8, state[2], hist, &sh_state);
     beta = sh_beta[0];
 #pragma unroll
     for (int i = 1; i < TOPK_MW_THREADS / 64; i++) beta = (sh_beta[i] <= beta) ? beta : sh_beta[i];
@@ -609,27 +612,37 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     }
 }
 
-// a row's workspace in dwords: slices[4][n_wg][256], four states, above[3][n_wg] (+ padding to
+// a row's workspace in dwords: slices[4][sl][256], four states, above[3][n_wg] (+ padding to
 // keep the rows 8-byte aligned)
-static size_t topk_mw_row_dwords(int64_t n_wg) { return (size_t)4 * n_wg * 256 + 2 * 4 + (size_t)((3 * n_wg + 1) & ~(int64_t)1); }
+static size_t topk_mw_row_dwords(int64_t n_wg, int64_t sl) { return (size_t)4 * sl * 256 + 2 * 4 + (size_t)((3 * n_wg + 1) & ~(int64_t)1); }
+static int64_t topk_mw_wgs(int64_t n) { return (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS; }
+// the banded select's layout: room for the approximate kernel's pass-0 slices
+static int64_t topk_mw_band_sl(int64_t n) {
+    const int64_t n_wg = topk_mw_wgs(n), n_s0 = indexer_approx_slots(n);
+    return n_wg > n_s0 ? n_wg : n_s0;
+}
+size_t topk_mw_band_row_dwords(int64_t n) { return topk_mw_row_dwords(topk_mw_wgs(n), topk_mw_band_sl(n)); }
 
+// enough for either layout
 size_t topk_mw_workspace_bytes(int batch, int64_t n) {
-    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
-    return (size_t)batch * topk_mw_row_dwords(n_wg) * sizeof(uint32_t);
+    return (size_t)batch * topk_mw_band_row_dwords(n) * sizeof(uint32_t);
 }
 
 int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
                               const float *beta_slots, int n_beta, int32_t *cand, int cap,
-                              IndexerBandRow *rows, hipStream_t s) {
-    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
+                              IndexerBandRow *rows, bool digit0_done, hipStream_t s) {
+    const int64_t n_wg = topk_mw_wgs(n);
     CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && n_beta <= TOPK_MW_THREADS,
                   "topk_band_classify: n %lld out of range", (long long)n);
-    const size_t ws_row = topk_mw_row_dwords(n_wg);
+    const int sl = (int)topk_mw_band_sl(n);
+    const int n_s0 = digit0_done ? indexer_approx_slots(n) : (int)n_wg;
+    CWICK_REQUIRE(n_s0 <= 2 * TOPK_MW_MAX_WGS, "topk_band_classify: %d first-digit slices", n_s0);
+    const size_t ws_row = topk_mw_band_row_dwords(n);
     const dim3 grid((unsigned)n_wg, (unsigned)batch);
-    for (int pass = 0; pass < 3; pass++)
-        topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row);
+    for (int pass = digit0_done ? 1 : 0; pass < 3; pass++)
+        topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row, sl, n_s0);
     topk_mw_classify_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, beta_slots,
-                                                            n_beta, cand, cap, rows);
+                                                            n_beta, cand, cap, rows, sl);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }
@@ -640,16 +653,16 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     CWICK_REQUIRE(batch >= 1 && batch <= 65535, "topk: batch %d", batch);
     CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
-    const int64_t n_wg = (n + TOPK_MW_KEYS - 1) / TOPK_MW_KEYS;
+    const int64_t n_wg = topk_mw_wgs(n);
     if (n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS) {
-        const size_t ws_row = topk_mw_row_dwords(n_wg);             // dwords: slices, then four states
+        const size_t ws_row = topk_mw_row_dwords(n_wg, n_wg);       // dwords: slices, four states, above counts
         uint32_t *ws = (uint32_t *)workspace(s, (size_t)batch * ws_row * sizeof(uint32_t));
         CWICK_REQUIRE(ws, "topk: workspace allocation failed");
         const dim3 grid((unsigned)n_wg, (unsigned)batch);
         ProfScope ps(CWICK_HIP_PROF_TOPK, s);
         for (int pass = 0; pass < 4; pass++)
-            topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row);
-        topk_mw_emit_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, out_idx);
+            topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row, (int)n_wg, (int)n_wg);
+        topk_mw_emit_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, (int)n_wg, out_idx);
         CWICK_HIP_CALL(hipGetLastError());
         return 1;
     }
