@@ -87,9 +87,12 @@ __host__ __device__ inline bool indexer_band_failed(const IndexerBandRow &r, int
 inline bool indexer_band_applies(int64_t n_keys, int64_t k, int n_idx_heads) {
     return n_keys >= 16384 && n_keys <= 131072 && k < n_keys && n_idx_heads >= 1 && n_idx_heads <= 64;
 }
+// indexer and top-k in one: `scores` is scratch (its contents afterwards are not scores), the
+// selected indices of every row go to out_idx[batch][k] in ascending order
 int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
-                          const float *w, int n_idx_heads, int64_t k, float *scores, hipStream_t s);
+                          const float *w, int n_idx_heads, int64_t k, float *scores, int32_t *out_idx,
+                          hipStream_t s);
 // the exact kernel for the rows whose band failed (returns at once for the others)
 int launch_indexer_scores_rows(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                                int64_t kscale_bstride, int batch, int64_t n_keys,
@@ -104,7 +107,13 @@ size_t topk_mw_workspace_bytes(int batch, int64_t n);
 size_t topk_mw_band_row_dwords(int64_t n);
 int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
                               const float *beta_slots, int n_beta, int32_t *cand, int cap,
-                              IndexerBandRow *rows, bool digit0_done, hipStream_t s);
+                              IndexerBandRow *rows, uint32_t *hi_count, bool digit0_done, hipStream_t s);
+// The end of the banded select, after the candidates have their exact scores: ranks the
+// candidates, writes the selected indices of every row that fitted the band, and runs the
+// plain select for the rows that did not (their scores are the exact kernel's by then).
+// hi_count: [batch][64] dwords, filled by launch_topk_band_classify.
+int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand, int cap,
+                            const IndexerBandRow *rows, uint32_t *hi_count, int32_t *out_idx, hipStream_t s);
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s);
 int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,

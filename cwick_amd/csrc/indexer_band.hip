@@ -26,9 +26,9 @@
 //      the second -inf, the rest (a few hundred of 65536) are candidates.
 //   4. indexer_rescore_kernel: the reference's arithmetic, instruction for instruction as in
 //      indexer.hip, for the candidates only, spread over heads so that it takes microseconds.
-//   5. the exact top-k over the patched scores returns the reference's indices: the +inf keys
-//      are fewer than k and all belong to the selection, the -inf keys do not, and among the
-//      candidates the order is that of their exact scores and indices.
+//   5. the selection is the +inf keys (fewer than k, all selected) and the best k - (their number)
+//      candidates by exact score, ties to the smaller index: one workgroup per row ranks the
+//      candidates and an ordered pass writes the indices (topk.hip).
 // Whenever a row does not fit this (more candidates than the list holds, a bound that is not
 // finite, NaN where T should be), the exact kernel runs for that row after all: it is always
 // launched and returns at once for rows that went well.
@@ -350,8 +350,9 @@ int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_
 
 int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
-                          const float *w, int n_idx_heads, int64_t k, float *scores, hipStream_t s) {
-    CWICK_REQUIRE(keys && kscale && q_idx && w && scores, "indexer_banded: null pointer");
+                          const float *w, int n_idx_heads, int64_t k, float *scores, int32_t *out_idx,
+                          hipStream_t s) {
+    CWICK_REQUIRE(keys && kscale && q_idx && w && scores && out_idx, "indexer_banded: null pointer");
     CWICK_REQUIRE(indexer_band_applies(n_keys, k, n_idx_heads), "indexer_banded: shape out of range");
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
                   "indexer_banded: keys and q must be 16-byte aligned");
@@ -361,26 +362,32 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     const size_t topk_bytes = topk_mw_workspace_bytes(batch, n_keys);
     size_t off_beta = (topk_bytes + 255) & ~(size_t)255;
     size_t off_rows = off_beta + (((size_t)batch * n_wg * sizeof(float) + 255) & ~(size_t)255);
-    size_t off_cand = off_rows + (((size_t)batch * sizeof(IndexerBandRow) + 255) & ~(size_t)255);
+    size_t off_hi = off_rows + (((size_t)batch * sizeof(IndexerBandRow) + 255) & ~(size_t)255);
+    size_t off_cand = off_hi + (size_t)batch * 64 * sizeof(uint32_t);
     const size_t total = off_cand + (size_t)batch * cap * sizeof(int32_t);
     char *ws = (char *)workspace(s, total);
     CWICK_REQUIRE(ws, "indexer_banded: workspace allocation failed");
     float *beta_slots = (float *)(ws + off_beta);
     IndexerBandRow *rows = (IndexerBandRow *)(ws + off_rows);
+    uint32_t *hi_count = (uint32_t *)(ws + off_hi);
     int32_t *cand = (int32_t *)(ws + off_cand);
+    {
     ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
     if (!launch_indexer_approx(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w, n_idx_heads,
                                scores, beta_slots, rows, (uint32_t *)ws, topk_mw_band_row_dwords(n_keys), s))
         return 0;
     if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows,
-                                   true, s))
+                                   hi_count, true, s))
         return 0;
     indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
         keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores);
     CWICK_HIP_CALL(hipGetLastError());
     // rows that did not fit the band take the exact kernel after all
-    return launch_indexer_scores_rows(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
-                                      n_idx_heads, scores, rows, cap, s);
+    if (!launch_indexer_scores_rows(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
+                                    n_idx_heads, scores, rows, cap, s))
+        return 0;
+    }
+    return launch_topk_band_finish(scores, batch, n_keys, k, cand, cap, rows, hi_count, out_idx, s);
 }
 
 }  // namespace cwick

@@ -558,13 +558,14 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale, int64_t
     }();
     if (!exact_only && indexer_band_applies(n_keys, topk, n_idx_heads)) {
         if (!launch_indexer_banded(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
-                                   q_idx, w, n_idx_heads, topk, scores_tmp, s))
+                                   q_idx, w, n_idx_heads, topk, scores_tmp, sel_out, s))
             return 0;
-    } else if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch,
-                                      n_keys, q_idx, w, n_idx_heads, scores_tmp, s)) {
-        return 0;
+    } else {
+        if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch,
+                                   n_keys, q_idx, w, n_idx_heads, scores_tmp, s))
+            return 0;
+        if (!launch_topk(scores_tmp, batch, n_keys, topk, sel_out, s)) return 0;
     }
-    if (!launch_topk(scores_tmp, batch, n_keys, topk, sel_out, s)) return 0;
     // rows past min(topk, n_keys) are -1 and are skipped by the attention kernel
     return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_keys, batch,
                              sel_out, topk, q, n_heads, scale, out, s);

@@ -56,7 +56,9 @@ __device__ __forceinline__ uint32_t block_exscan(uint32_t v, uint32_t *sh_wave, 
 
 __global__ void __launch_bounds__(TOPK_THREADS)
 topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
-                  int32_t *__restrict__ out) {
+                  int32_t *__restrict__ out,
+                  const IndexerBandRow *__restrict__ rows, int cap) {   // optional: only the rows whose band failed
+    if (rows && !indexer_band_failed(rows[blockIdx.x], cap)) return;
     // 16 copies of the histogram, picked by lane, so that the lanes of a wave
     // that hit one digit (scores cluster in a few exponent buckets) do not all
     // serialise on one LDS word
@@ -539,7 +541,8 @@ __global__ void __launch_bounds__(TOPK_MW_THREADS)
 topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
                         const uint32_t *__restrict__ ws, size_t ws_row,
                         const float *__restrict__ beta_slots, int n_beta,
-                        int32_t *__restrict__ cand, int cap, IndexerBandRow *__restrict__ rows, int sl) {
+                        int32_t *__restrict__ cand, int cap, IndexerBandRow *__restrict__ rows, int sl,
+                        uint32_t *__restrict__ hi_count) {   // [row][TOPK_MW_MAX_WGS]: keys set to +inf per workgroup
     __shared__ uint32_t hist[256];
     __shared__ TopkMwState sh_state;
     __shared__ float sh_beta[TOPK_MW_THREADS / 64];
@@ -582,15 +585,15 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     // candidates take a place in the workgroup first (LDS counter), the workgroup then takes its
     // run of the row's list with one atomic: a few hundred returning atomics on one address from
     // all over the chip would queue up behind each other
-    uint32_t *wg_count = &hist[0], *wg_base = &hist[1];          // the pick is done with hist
-    if (tid == 0) *wg_count = 0u;
+    uint32_t *wg_count = &hist[0], *wg_base = &hist[1], *wg_hi = &hist[2];   // the pick is done with hist
+    if (tid == 0) *wg_count = 0u, *wg_hi = 0u;
     __syncthreads();
-    uint32_t is_cand = 0u;
+    uint32_t is_cand = 0u, n_hi = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_MW_EPT; j++) {
         const int64_t i = base + j * TOPK_MW_THREADS + tid;
         if (i < n) {
-            if (v[j] > hi) sc[i] = INFINITY;
+            if (v[j] > hi) sc[i] = INFINITY, n_hi++;
             else if (v[j] < lo) sc[i] = -INFINITY;
             else is_cand |= 1u << j;
         }
@@ -598,8 +601,12 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     uint32_t my_first = 0u;
     const uint32_t mine = (uint32_t)__builtin_popcount(is_cand);
     if (mine) my_first = atomicAdd(wg_count, mine);
+    if (n_hi) atomicAdd(wg_hi, n_hi);
     __syncthreads();
-    if (tid == 0) *wg_base = *wg_count ? atomicAdd(&rows[row].n_cand, *wg_count) : 0u;
+    if (tid == 0) {
+        *wg_base = *wg_count ? atomicAdd(&rows[row].n_cand, *wg_count) : 0u;
+        hi_count[(size_t)row * TOPK_MW_MAX_WGS + wg] = *wg_hi;
+    }
     __syncthreads();
     if (mine) {
         uint32_t slot = *wg_base + my_first;
@@ -610,6 +617,154 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
                 slot++;
             }
     }
+}
+
+// ---- the end of the banded select: no second radix select over the whole row ----
+// After the classify kernel and the exact rescoring a row consists of keys that are certainly
+// selected (+inf, hi_count[w] of them in workgroup w's stretch), keys that are certainly not
+// (-inf) and at most `cap` candidates with their exact scores.  The selection is the +inf keys
+// and the best need = k - (number of +inf keys) candidates, ties to the smaller index as
+// everywhere.  One workgroup per row ranks the candidates on the 64-bit key (order key of the
+// score, then the inverted index: all distinct, so there are no ties left to count), turns
+// the chosen ones into +inf and the others into -inf and adds them to hi_count; the emit
+// kernel then only has to write out the +inf keys in index order.
+constexpr int TOPK_BAND_THREADS = 1024;
+constexpr int TOPK_BAND_EPT = CWICK_INDEXER_BAND_CAP / TOPK_BAND_THREADS;     // 4
+__global__ void __launch_bounds__(TOPK_BAND_THREADS)
+topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
+                      const int32_t *__restrict__ cand, int cap,
+                      const IndexerBandRow *__restrict__ rows, uint32_t *__restrict__ hi_count) {
+    __shared__ uint32_t hist8[256 * 8];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t sh_digit, sh_remaining, sh_hi;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const IndexerBandRow st = rows[row];
+    if (indexer_band_failed(st, cap)) return;
+    float *sc = scores + (size_t)row * n;
+    uint32_t *hc = hi_count + (size_t)row * TOPK_MW_MAX_WGS;
+    const int n_cand = (int)st.n_cand;
+    if (tid == 0) sh_hi = 0u;
+    __syncthreads();
+    if (tid < n_wg) atomicAdd(&sh_hi, hc[tid]);
+    int32_t idx[TOPK_BAND_EPT];
+    uint64_t comp[TOPK_BAND_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_BAND_EPT; j++) {
+        const int c = tid + TOPK_BAND_THREADS * j;
+        idx[j] = c < n_cand ? cand[(size_t)row * cap + c] : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < TOPK_BAND_EPT; j++)
+        comp[j] = idx[j] >= 0 ? ((uint64_t)topk_key(sc[idx[j]]) << 32) | (uint32_t)~(uint32_t)idx[j] : 0ull;
+    __syncthreads();
+    const int64_t want = k - (int64_t)sh_hi;
+    const uint32_t need = want <= 0 ? 0u : (want < n_cand ? (uint32_t)want : (uint32_t)n_cand);
+    uint64_t prefix = 0ull, mask = 0ull;
+    uint32_t remaining = need;
+    if (need > 0u) {
+        for (int shift = 56; shift >= 0; shift -= 8) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) hist8[tid * 2 + j] = 0u;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < TOPK_BAND_EPT; j++)
+                if (idx[j] >= 0 && (comp[j] & mask) == prefix)
+                    atomicAdd(&hist8[(uint32_t)((comp[j] >> shift) & 0xFFull) * 8 + (tid & 7)], 1u);
+            __syncthreads();
+            if (tid < 256) {
+                uint32_t c = 0u;
+#pragma unroll
+                for (int j = 0; j < 8; j++) c += hist8[tid * 8 + ((j + tid) & 7)];
+                hist[tid] = c;
+            }
+            __syncthreads();
+            if (tid < 64) {
+                // walk the 256 buckets from the largest digit down; lane b owns buckets 255-4b .. 252-4b
+                uint32_t c[4], sum = 0u;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    c[j] = hist[255 - (tid * 4 + j)];
+                    sum += c[j];
+                }
+                uint32_t inc = sum;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {
+                    uint32_t t = __shfl_up(inc, o, 64);
+                    if (tid >= o) inc += t;
+                }
+                uint32_t before = inc - sum;   // elements in strictly larger buckets
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (before < remaining && remaining <= before + c[j]) {
+                        sh_digit = (uint32_t)(255 - (tid * 4 + j));
+                        sh_remaining = remaining - before;
+                    }
+                    before += c[j];
+                }
+            }
+            __syncthreads();
+            prefix |= (uint64_t)sh_digit << shift;
+            remaining = sh_remaining;
+            mask |= 0xFFull << shift;
+            __syncthreads();
+        }
+    }
+    // prefix is now the need-th largest key itself
+#pragma unroll
+    for (int j = 0; j < TOPK_BAND_EPT; j++)
+        if (idx[j] >= 0) {
+            const bool take = need > 0u && comp[j] >= prefix;
+            sc[idx[j]] = take ? INFINITY : -INFINITY;
+            if (take) atomicAdd(&hc[idx[j] / TOPK_MW_KEYS], 1u);
+        }
+}
+
+// writes the indices of a row's +inf keys in ascending order; workgroup w starts after the
+// hi_count of the workgroups before it
+__global__ void __launch_bounds__(TOPK_MW_THREADS)
+topk_band_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
+                      const IndexerBandRow *__restrict__ rows, int cap,
+                      const uint32_t *__restrict__ hi_count, int32_t *__restrict__ out) {
+    __shared__ uint32_t sh_before;
+    __shared__ uint32_t sh_cnt[TOPK_MW_EPT][TOPK_MW_THREADS / 64];
+    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (indexer_band_failed(rows[row], cap)) return;
+    const float *sc = scores + (size_t)row * n;
+    int32_t *dst = out + (size_t)row * k;
+    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
+    float v[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        const int64_t i = base + j * TOPK_MW_THREADS + tid;
+        v[j] = i < n ? sc[i] : 0.0f;
+    }
+    if (tid == 0) sh_before = 0u;
+    __syncthreads();
+    if (tid < wg) atomicAdd(&sh_before, hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid]);
+    // element (j, tid) is index base + 256 j + tid: the order of the workgroup is (j, wave, lane)
+    uint64_t m[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++) {
+        m[j] = __ballot(v[j] == INFINITY);
+        if (lane == 0) sh_cnt[j][wave] = (uint32_t)__builtin_popcountll(m[j]);
+    }
+    __syncthreads();
+    uint32_t run = sh_before, my_pos[TOPK_MW_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++)
+#pragma unroll
+        for (int w = 0; w < TOPK_MW_THREADS / 64; w++) {
+            if (w == wave) my_pos[j] = run;
+            run += sh_cnt[j][w];
+        }
+    const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int j = 0; j < TOPK_MW_EPT; j++)
+        if ((m[j] >> lane) & 1) {
+            const uint32_t pos = my_pos[j] + (uint32_t)__builtin_popcountll(m[j] & lt);
+            if (pos < (uint32_t)k) dst[pos] = (int32_t)(base + j * TOPK_MW_THREADS + tid);
+        }
 }
 
 // a row's workspace in dwords: slices[4][sl][256], four states, above[3][n_wg] (+ padding to
@@ -630,7 +785,7 @@ size_t topk_mw_workspace_bytes(int batch, int64_t n) {
 
 int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, uint32_t *ws,
                               const float *beta_slots, int n_beta, int32_t *cand, int cap,
-                              IndexerBandRow *rows, bool digit0_done, hipStream_t s) {
+                              IndexerBandRow *rows, uint32_t *hi_count, bool digit0_done, hipStream_t s) {
     const int64_t n_wg = topk_mw_wgs(n);
     CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && n_beta <= TOPK_MW_THREADS,
                   "topk_band_classify: n %lld out of range", (long long)n);
@@ -642,7 +797,23 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
     for (int pass = digit0_done ? 1 : 0; pass < 3; pass++)
         topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row, sl, n_s0);
     topk_mw_classify_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, beta_slots,
-                                                            n_beta, cand, cap, rows, sl);
+                                                            n_beta, cand, cap, rows, sl, hi_count);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand, int cap,
+                            const IndexerBandRow *rows, uint32_t *hi_count, int32_t *out_idx, hipStream_t s) {
+    static_assert(TOPK_BAND_EPT * TOPK_BAND_THREADS == CWICK_INDEXER_BAND_CAP, "the pick kernel holds the whole list");
+    const int64_t n_wg = topk_mw_wgs(n);
+    CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && cap == CWICK_INDEXER_BAND_CAP && k < n,
+                  "topk_band_finish: n %lld out of range", (long long)n);
+    ProfScope ps(CWICK_HIP_PROF_TOPK, s);
+    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cap, rows, hi_count);
+    topk_band_emit_kernel<<<dim3((unsigned)n_wg, (unsigned)batch), TOPK_MW_THREADS, 0, s>>>(scores, n, k, rows, cap,
+                                                                                              hi_count, out_idx);
+    // rows that did not fit the band: their scores are the exact kernel's, one workgroup each
+    topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx, rows, cap);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }
@@ -671,7 +842,7 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
         if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)
             topk_radix_reg_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
         else
-            topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+            topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx, nullptr, 0);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
