@@ -112,8 +112,10 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
 // candidates, writes the selected indices of every row that fitted the band, and runs the
 // plain select for the rows that did not (their scores are the exact kernel's by then).
 // hi_count: [batch][64] dwords, filled by launch_topk_band_classify.
-int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand, int cap,
-                            const IndexerBandRow *rows, uint32_t *hi_count, int32_t *out_idx, hipStream_t s);
+// cand_score: [batch][cap], the exact score of every list entry (what the rescoring wrote).
+int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand,
+                            const float *cand_score, int cap, const IndexerBandRow *rows, uint32_t *hi_count,
+                            int32_t *out_idx, hipStream_t s);
 int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                 hipStream_t s);
 int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,

@@ -252,7 +252,8 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
                        int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
                        const uint16_t *__restrict__ q, const float *__restrict__ w, int ih,
                        const int32_t *__restrict__ cand, int cap,
-                       const IndexerBandRow *__restrict__ rows, float *__restrict__ scores) {
+                       const IndexerBandRow *__restrict__ rows, float *__restrict__ scores,
+                       float *__restrict__ cand_score) {   // [batch][cap]: the same scores in list order
     __shared__ float terms[16][65];
     const int b = blockIdx.y, tid = threadIdx.x;
     const IndexerBandRow st = rows[b];
@@ -325,6 +326,7 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
         float s = 0.0f;
         for (int h = 0; h < ih; h++) s = s + terms[tid][h];
         scores[(size_t)b * n_keys + cand[(size_t)b * cap + c0 + tid]] = s;
+        cand_score[(size_t)b * cap + c0 + tid] = s;
     }
 }
 
@@ -358,19 +360,21 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
                   "indexer_banded: keys and q must be 16-byte aligned");
     const int n_wg = indexer_approx_slots(n_keys);
     constexpr int cap = CWICK_INDEXER_BAND_CAP;
-    // workspace: [the top-k's slices and states][beta slots][row states][candidate lists]
+    // workspace: [the top-k's slices and states][beta slots][row states][+inf counts][candidate lists][their exact scores]
     const size_t topk_bytes = topk_mw_workspace_bytes(batch, n_keys);
     size_t off_beta = (topk_bytes + 255) & ~(size_t)255;
     size_t off_rows = off_beta + (((size_t)batch * n_wg * sizeof(float) + 255) & ~(size_t)255);
     size_t off_hi = off_rows + (((size_t)batch * sizeof(IndexerBandRow) + 255) & ~(size_t)255);
     size_t off_cand = off_hi + (size_t)batch * 64 * sizeof(uint32_t);
-    const size_t total = off_cand + (size_t)batch * cap * sizeof(int32_t);
+    size_t off_cs = off_cand + (size_t)batch * cap * sizeof(int32_t);
+    const size_t total = off_cs + (size_t)batch * cap * sizeof(float);
     char *ws = (char *)workspace(s, total);
     CWICK_REQUIRE(ws, "indexer_banded: workspace allocation failed");
     float *beta_slots = (float *)(ws + off_beta);
     IndexerBandRow *rows = (IndexerBandRow *)(ws + off_rows);
     uint32_t *hi_count = (uint32_t *)(ws + off_hi);
     int32_t *cand = (int32_t *)(ws + off_cand);
+    float *cand_score = (float *)(ws + off_cs);
     {
     ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
     if (!launch_indexer_approx(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w, n_idx_heads,
@@ -380,14 +384,14 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
                                    hi_count, true, s))
         return 0;
     indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
-        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores);
+        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores, cand_score);
     CWICK_HIP_CALL(hipGetLastError());
     // rows that did not fit the band take the exact kernel after all
     if (!launch_indexer_scores_rows(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
                                     n_idx_heads, scores, rows, cap, s))
         return 0;
     }
-    return launch_topk_band_finish(scores, batch, n_keys, k, cand, cap, rows, hi_count, out_idx, s);
+    return launch_topk_band_finish(scores, batch, n_keys, k, cand, cand_score, cap, rows, hi_count, out_idx, s);
 }
 
 }  // namespace cwick

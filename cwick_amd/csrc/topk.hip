@@ -624,96 +624,151 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
 // selected (+inf, hi_count[w] of them in workgroup w's stretch), keys that are certainly not
 // (-inf) and at most `cap` candidates with their exact scores.  The selection is the +inf keys
 // and the best need = k - (number of +inf keys) candidates, ties to the smaller index as
-// everywhere.  One workgroup per row ranks the candidates on the 64-bit key (order key of the
-// score, then the inverted index: all distinct, so there are no ties left to count), turns
-// the chosen ones into +inf and the others into -inf and adds them to hi_count; the emit
-// kernel then only has to write out the +inf keys in index order.
+// everywhere.  One workgroup per row ranks the candidates (a radix select on the order keys of
+// their scores, and, if the need-th key has ties that do not all fit, a second one on the
+// inverted indices of the tied), turns the chosen ones into +inf and the others into -inf and
+// adds them to hi_count; the emit kernel then only has to write out the +inf keys in index
+// order.
 constexpr int TOPK_BAND_THREADS = 1024;
 constexpr int TOPK_BAND_EPT = CWICK_INDEXER_BAND_CAP / TOPK_BAND_THREADS;     // 4
+
+struct TopkBandShared {
+    uint32_t hist[256];
+    uint32_t mn[TOPK_BAND_THREADS / 64], mx[TOPK_BAND_THREADS / 64], cnt[TOPK_BAND_THREADS / 64];
+    uint32_t digit, remaining, eq;
+};
+
+// Radix select inside one workgroup over up to four 32-bit values per thread (`act` marks
+// the live ones): T = the need-th largest, r = how many of the values equal to T belong to
+// the need largest, e = how many values equal T.  1 <= need <= number of live values.  The
+// values of a candidate list agree in their leading bits (scores from a narrow band, indices
+// from one row), and digits that all values share would put every LDS atomic on one word: the
+// passes start at the first byte in which the largest and the smallest value differ.
+__device__ __forceinline__ void topk_band_select(const uint32_t (&val)[TOPK_BAND_EPT], uint32_t act, uint32_t need,
+                                                 TopkBandShared &sh, uint32_t &T, uint32_t &r, uint32_t &e) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t mn = 0xFFFFFFFFu, mx = 0u, cnt = (uint32_t)__builtin_popcount(act);
+#pragma unroll
+    for (int j = 0; j < TOPK_BAND_EPT; j++)
+        if (act >> j & 1u) {
+            mn = val[j] < mn ? val[j] : mn;
+            mx = val[j] > mx ? val[j] : mx;
+        }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t a = __shfl_xor(mn, o, 64), b = __shfl_xor(mx, o, 64);
+        mn = a < mn ? a : mn;
+        mx = b > mx ? b : mx;
+        cnt += __shfl_xor(cnt, o, 64);
+    }
+    if (lane == 0) sh.mn[wave] = mn, sh.mx[wave] = mx, sh.cnt[wave] = cnt;
+    __syncthreads();
+    cnt = 0u;
+#pragma unroll
+    for (int w = 0; w < TOPK_BAND_THREADS / 64; w++) {
+        mn = sh.mn[w] < mn ? sh.mn[w] : mn;
+        mx = sh.mx[w] > mx ? sh.mx[w] : mx;
+        cnt += sh.cnt[w];
+    }
+    const uint32_t diff = mn ^ mx;
+    const int passes = diff ? (31 - __builtin_clz(diff)) / 8 + 1 : 0;
+    uint32_t mask = passes >= 4 ? 0u : 0xFFFFFFFFu << (8 * passes);
+    uint32_t prefix = mx & mask, remaining = need;
+    e = cnt;                                              // all values equal: every one is a tie
+    for (int p = passes - 1; p >= 0; p--) {
+        const int shift = 8 * p;
+        if (tid < 256) sh.hist[tid] = 0u;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < TOPK_BAND_EPT; j++)
+            if ((act >> j & 1u) && (val[j] & mask) == prefix) atomicAdd(&sh.hist[(val[j] >> shift) & 0xFFu], 1u);
+        __syncthreads();
+        if (tid < 64) {
+            // walk the 256 buckets from the largest digit down; lane b owns buckets 255-4b .. 252-4b
+            uint32_t c[4], sum = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                c[j] = sh.hist[255 - (tid * 4 + j)];
+                sum += c[j];
+            }
+            uint32_t inc = sum;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                uint32_t t = __shfl_up(inc, o, 64);
+                if (tid >= o) inc += t;
+            }
+            uint32_t before = inc - sum;   // values in strictly larger buckets
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (before < remaining && remaining <= before + c[j]) {
+                    sh.digit = (uint32_t)(255 - (tid * 4 + j));
+                    sh.remaining = remaining - before;
+                    sh.eq = c[j];
+                }
+                before += c[j];
+            }
+        }
+        __syncthreads();
+        prefix |= sh.digit << shift;
+        remaining = sh.remaining;
+        e = sh.eq;
+        mask |= 0xFFu << shift;
+    }
+    __syncthreads();                                      // sh is free again
+    T = prefix;
+    r = remaining;
+}
+
 __global__ void __launch_bounds__(TOPK_BAND_THREADS)
 topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
-                      const int32_t *__restrict__ cand, int cap,
+                      const int32_t *__restrict__ cand, const float *__restrict__ cand_score, int cap,
                       const IndexerBandRow *__restrict__ rows, uint32_t *__restrict__ hi_count) {
-    __shared__ uint32_t hist8[256 * 8];
-    __shared__ uint32_t hist[256];
-    __shared__ uint32_t sh_digit, sh_remaining, sh_hi;
+    __shared__ TopkBandShared sh;
+    __shared__ uint32_t sh_hi;
     const int row = blockIdx.x, tid = threadIdx.x;
+    // the whole list is loaded whatever its length (the thread count times four is its
+    // capacity): these loads then travel together with the row state they would depend on
+    int32_t idx[TOPK_BAND_EPT];
+    float val[TOPK_BAND_EPT];
+#pragma unroll
+    for (int j = 0; j < TOPK_BAND_EPT; j++) {
+        idx[j] = cand[(size_t)row * cap + tid + TOPK_BAND_THREADS * j];
+        val[j] = cand_score[(size_t)row * cap + tid + TOPK_BAND_THREADS * j];
+    }
+    uint32_t *hc = hi_count + (size_t)row * TOPK_MW_MAX_WGS;
+    const uint32_t hi_part = tid < n_wg ? hc[tid] : 0u;
     const IndexerBandRow st = rows[row];
     if (indexer_band_failed(st, cap)) return;
     float *sc = scores + (size_t)row * n;
-    uint32_t *hc = hi_count + (size_t)row * TOPK_MW_MAX_WGS;
     const int n_cand = (int)st.n_cand;
     if (tid == 0) sh_hi = 0u;
     __syncthreads();
-    if (tid < n_wg) atomicAdd(&sh_hi, hc[tid]);
-    int32_t idx[TOPK_BAND_EPT];
-    uint64_t comp[TOPK_BAND_EPT];
+    if (tid < n_wg) atomicAdd(&sh_hi, hi_part);
+    uint32_t key[TOPK_BAND_EPT], inv[TOPK_BAND_EPT], live = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++) {
-        const int c = tid + TOPK_BAND_THREADS * j;
-        idx[j] = c < n_cand ? cand[(size_t)row * cap + c] : -1;
+        key[j] = topk_key(val[j]);
+        inv[j] = ~(uint32_t)idx[j];
+        if (tid + TOPK_BAND_THREADS * j < n_cand) live |= 1u << j;
     }
-#pragma unroll
-    for (int j = 0; j < TOPK_BAND_EPT; j++)
-        comp[j] = idx[j] >= 0 ? ((uint64_t)topk_key(sc[idx[j]]) << 32) | (uint32_t)~(uint32_t)idx[j] : 0ull;
     __syncthreads();
     const int64_t want = k - (int64_t)sh_hi;
     const uint32_t need = want <= 0 ? 0u : (want < n_cand ? (uint32_t)want : (uint32_t)n_cand);
-    uint64_t prefix = 0ull, mask = 0ull;
-    uint32_t remaining = need;
-    if (need > 0u) {
-        for (int shift = 56; shift >= 0; shift -= 8) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) hist8[tid * 2 + j] = 0u;
-            __syncthreads();
+    uint32_t T = 0u, r = 0u, e = 0u, T2 = 0u;
+    if (need > 0u) {                                            // uniform
+        topk_band_select(key, live, need, sh, T, r, e);
+        if (r < e) {                                            // uniform: ties at T, the smaller indices win
+            uint32_t tied = 0u, r2, e2;
 #pragma unroll
             for (int j = 0; j < TOPK_BAND_EPT; j++)
-                if (idx[j] >= 0 && (comp[j] & mask) == prefix)
-                    atomicAdd(&hist8[(uint32_t)((comp[j] >> shift) & 0xFFull) * 8 + (tid & 7)], 1u);
-            __syncthreads();
-            if (tid < 256) {
-                uint32_t c = 0u;
-#pragma unroll
-                for (int j = 0; j < 8; j++) c += hist8[tid * 8 + ((j + tid) & 7)];
-                hist[tid] = c;
-            }
-            __syncthreads();
-            if (tid < 64) {
-                // walk the 256 buckets from the largest digit down; lane b owns buckets 255-4b .. 252-4b
-                uint32_t c[4], sum = 0u;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    c[j] = hist[255 - (tid * 4 + j)];
-                    sum += c[j];
-                }
-                uint32_t inc = sum;
-#pragma unroll
-                for (int o = 1; o < 64; o <<= 1) {
-                    uint32_t t = __shfl_up(inc, o, 64);
-                    if (tid >= o) inc += t;
-                }
-                uint32_t before = inc - sum;   // elements in strictly larger buckets
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    if (before < remaining && remaining <= before + c[j]) {
-                        sh_digit = (uint32_t)(255 - (tid * 4 + j));
-                        sh_remaining = remaining - before;
-                    }
-                    before += c[j];
-                }
-            }
-            __syncthreads();
-            prefix |= (uint64_t)sh_digit << shift;
-            remaining = sh_remaining;
-            mask |= 0xFFull << shift;
-            __syncthreads();
+                if ((live >> j & 1u) && key[j] == T) tied |= 1u << j;
+            topk_band_select(inv, tied, r, sh, T2, r2, e2);
         }
     }
-    // prefix is now the need-th largest key itself
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++)
-        if (idx[j] >= 0) {
-            const bool take = need > 0u && comp[j] >= prefix;
+        if (live >> j & 1u) {
+            const bool take = need > 0u && (key[j] > T || (key[j] == T && inv[j] >= T2));
             sc[idx[j]] = take ? INFINITY : -INFINITY;
             if (take) atomicAdd(&hc[idx[j] / TOPK_MW_KEYS], 1u);
         }
@@ -729,19 +784,22 @@ topk_band_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     __shared__ uint32_t sh_cnt[TOPK_MW_EPT][TOPK_MW_THREADS / 64];
     const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (indexer_band_failed(rows[row], cap)) return;
     const float *sc = scores + (size_t)row * n;
     int32_t *dst = out + (size_t)row * k;
     const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
-    float v[TOPK_MW_EPT];
+    float v[TOPK_MW_EPT];                       // all loads first: one round trip
 #pragma unroll
     for (int j = 0; j < TOPK_MW_EPT; j++) {
         const int64_t i = base + j * TOPK_MW_THREADS + tid;
-        v[j] = i < n ? sc[i] : 0.0f;
+        const int64_t ic = i < n ? i : n - 1;
+        v[j] = sc[ic];
+        if (i >= n) v[j] = 0.0f;
     }
+    const uint32_t before_part = tid < wg ? hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid] : 0u;
+    if (indexer_band_failed(rows[row], cap)) return;
     if (tid == 0) sh_before = 0u;
     __syncthreads();
-    if (tid < wg) atomicAdd(&sh_before, hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid]);
+    if (tid < wg) atomicAdd(&sh_before, before_part);
     // element (j, tid) is index base + 256 j + tid: the order of the workgroup is (j, wave, lane)
     uint64_t m[TOPK_MW_EPT];
 #pragma unroll
@@ -802,14 +860,15 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
     return 1;
 }
 
-int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand, int cap,
-                            const IndexerBandRow *rows, uint32_t *hi_count, int32_t *out_idx, hipStream_t s) {
+int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand,
+                            const float *cand_score, int cap, const IndexerBandRow *rows, uint32_t *hi_count,
+                            int32_t *out_idx, hipStream_t s) {
     static_assert(TOPK_BAND_EPT * TOPK_BAND_THREADS == CWICK_INDEXER_BAND_CAP, "the pick kernel holds the whole list");
     const int64_t n_wg = topk_mw_wgs(n);
     CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && cap == CWICK_INDEXER_BAND_CAP && k < n,
                   "topk_band_finish: n %lld out of range", (long long)n);
     ProfScope ps(CWICK_HIP_PROF_TOPK, s);
-    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cap, rows, hi_count);
+    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cand_score, cap, rows, hi_count);
     topk_band_emit_kernel<<<dim3((unsigned)n_wg, (unsigned)batch), TOPK_MW_THREADS, 0, s>>>(scores, n, k, rows, cap,
                                                                                               hi_count, out_idx);
     // rows that did not fit the band: their scores are the exact kernel's, one workgroup each
