@@ -349,6 +349,43 @@ def test_dsa_decode_small(hip, orc, n_keys, topk, ih):
     lat.free()
 
 
+@pytest.mark.parametrize("n_keys,topk,copies,take", [(20000, 512, 9, 4), (65536, 2048, 40, 1), (20000, 512, 6, 6)])
+def test_dsa_select_ties_at_the_threshold(hip, orc, n_keys, topk, copies, take):
+    """The key that closes the selection exists `copies` times (identical rows: identical exact
+    scores) and only `take` of the copies fit: the banded path has to rank its candidates by
+    score and then by index, as the reference does."""
+    say("[case] dsa select ties at the threshold", n_keys, topk, copies, take)
+    c = synth.cfg5_dsa(n_keys=n_keys, batch=2, ih=64, topk=topk, nh=128, seed=1300 + copies)
+    ikeys = c["ikeys"].copy(); ikscale = c["ikscale"].copy()
+    g = synth.rng(77 + copies)
+    for b in range(2):
+        sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], ikeys[b], ikscale[b], nthreads=0)
+        order = np.lexsort((np.arange(n_keys), -sc.astype(np.float64)))
+        # rank topk - take (0-based) is the first copy's rank: `take` copies end the selection
+        src = order[topk - take]
+        # overwrite keys that rank below the selection, at indices on both sides of src
+        dst = g.choice(order[topk + 50:], size=copies - 1, replace=False)
+        ikeys[b, dst] = ikeys[b, src]
+        ikscale[b, dst] = ikscale[b, src]
+    ik = hip.IndexKeys(2, n_keys)
+    lat = hip.LatentCache(2, n_keys)
+    for b in range(2):
+        ik.write(b, 0, ikeys[b], ikscale[b])
+        lat.write(b, 0, c["rows"][b], c["scales"][b])
+    out, sel = hip.dsa_decode(ik, lat, 0, 1, n_keys, c["q_idx"], c["w"], topk, c["q"], c["scale"])
+    for b in range(2):
+        sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], ikeys[b], ikscale[b], nthreads=0)
+        rsel = orc.topk_contract(sc, topk)
+        T = np.sort(sc)[::-1][topk - 1]
+        tied = int((sc == T).sum())
+        inside = int((sc[rsel[rsel >= 0]] == T).sum())
+        say("[parity] query %d: %d keys tie at the threshold, %d of them selected" % (b, tied, inside))
+        assert tied >= copies and inside < tied or take == copies
+        assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
+    ik.free()
+    lat.free()
+
+
 @pytest.mark.parametrize("kind", ["same", "two", "zero_w"])
 def test_dsa_select_degenerate(hip, orc, kind):
     """Selections where the error band of the approximate scores holds most keys (identical or
