@@ -54,11 +54,9 @@ __device__ __forceinline__ uint32_t block_exscan(uint32_t v, uint32_t *sh_wave, 
     return wave_off + inc - v;
 }
 
-__global__ void __launch_bounds__(TOPK_THREADS)
-topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
-                  int32_t *__restrict__ out,
-                  const IndexerBandRow *__restrict__ rows, int cap) {   // optional: only the rows whose band failed
-    if (rows && !indexer_band_failed(rows[blockIdx.x], cap)) return;
+// one row by one workgroup of TOPK_THREADS; sc and dst are the row's
+__device__ __forceinline__ void topk_radix_row(const float *__restrict__ sc, int64_t n, int64_t k,
+                                               int32_t *__restrict__ dst) {
     // 16 copies of the histogram, picked by lane, so that the lanes of a wave
     // that hit one digit (scores cluster in a few exponent buckets) do not all
     // serialise on one LDS word
@@ -66,8 +64,6 @@ topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     __shared__ uint32_t hist[256];
     __shared__ uint32_t sh_wave[TOPK_WAVES];
     __shared__ uint32_t sh_prefix, sh_remaining;
-    const float *sc = scores + (size_t)blockIdx.x * n;
-    int32_t *dst = out + (size_t)blockIdx.x * k;
     const int tid = threadIdx.x;
     const int64_t kk = k < n ? k : n;
 
@@ -159,6 +155,11 @@ topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
         out_base += take_total;
         eq_base += eq_total;
     }
+}
+
+__global__ void __launch_bounds__(TOPK_THREADS)
+topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int32_t *__restrict__ out) {
+    topk_radix_row(scores + (size_t)blockIdx.x * n, n, k, out + (size_t)blockIdx.x * k);
 }
 
 // ---- rows that fit the register file: n <= TOPK_THREADS * TOPK_EPT ----
@@ -722,7 +723,8 @@ __device__ __forceinline__ void topk_band_select(const uint32_t (&val)[TOPK_BAND
 __global__ void __launch_bounds__(TOPK_BAND_THREADS)
 topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
                       const int32_t *__restrict__ cand, const float *__restrict__ cand_score, int cap,
-                      const IndexerBandRow *__restrict__ rows, uint32_t *__restrict__ hi_count) {
+                      const IndexerBandRow *__restrict__ rows, uint32_t *__restrict__ hi_count,
+                      int32_t *__restrict__ out) {
     __shared__ TopkBandShared sh;
     __shared__ uint32_t sh_hi;
     const int row = blockIdx.x, tid = threadIdx.x;
@@ -738,8 +740,13 @@ topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg
     uint32_t *hc = hi_count + (size_t)row * TOPK_MW_MAX_WGS;
     const uint32_t hi_part = tid < n_wg ? hc[tid] : 0u;
     const IndexerBandRow st = rows[row];
-    if (indexer_band_failed(st, cap)) return;
     float *sc = scores + (size_t)row * n;
+    if (indexer_band_failed(st, cap)) {
+        // the row did not fit the band: its scores are the exact kernel's by now, and this
+        // workgroup selects from all of them (the emit kernel skips the row)
+        topk_radix_row(sc, n, k, out + (size_t)row * k);
+        return;
+    }
     const int n_cand = (int)st.n_cand;
     if (tid == 0) sh_hi = 0u;
     __syncthreads();
@@ -864,15 +871,14 @@ int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, cons
                             const float *cand_score, int cap, const IndexerBandRow *rows, uint32_t *hi_count,
                             int32_t *out_idx, hipStream_t s) {
     static_assert(TOPK_BAND_EPT * TOPK_BAND_THREADS == CWICK_INDEXER_BAND_CAP, "the pick kernel holds the whole list");
+    static_assert(TOPK_BAND_THREADS == TOPK_THREADS, "the pick kernel runs the one-workgroup select for rows off the band");
     const int64_t n_wg = topk_mw_wgs(n);
     CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && cap == CWICK_INDEXER_BAND_CAP && k < n,
                   "topk_band_finish: n %lld out of range", (long long)n);
     ProfScope ps(CWICK_HIP_PROF_TOPK, s);
-    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cand_score, cap, rows, hi_count);
+    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cand_score, cap, rows, hi_count, out_idx);
     topk_band_emit_kernel<<<dim3((unsigned)n_wg, (unsigned)batch), TOPK_MW_THREADS, 0, s>>>(scores, n, k, rows, cap,
                                                                                               hi_count, out_idx);
-    // rows that did not fit the band: their scores are the exact kernel's, one workgroup each
-    topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx, rows, cap);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }
@@ -901,7 +907,7 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
         if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)
             topk_radix_reg_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
         else
-            topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx, nullptr, 0);
+            topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
