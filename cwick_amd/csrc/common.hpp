@@ -93,11 +93,6 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
                           int64_t kscale_bstride, int batch, int64_t n_keys, const uint16_t *q_idx,
                           const float *w, int n_idx_heads, int64_t k, float *scores, int32_t *out_idx,
                           hipStream_t s);
-// the exact kernel for the rows whose band failed (returns at once for the others)
-int launch_indexer_scores_rows(const uint8_t *keys, const float *kscale, int64_t key_bstride,
-                               int64_t kscale_bstride, int batch, int64_t n_keys,
-                               const uint16_t *q_idx, const float *w, int n_idx_heads, float *scores,
-                               const IndexerBandRow *rows, int cap, hipStream_t s);
 // top-k machinery on approximate scores: finds T, then patches the scores (+inf / -inf / kept)
 // and lists the keys within 2 beta of T.  `ws` holds topk_mw_workspace_bytes() at its start.
 // With `digit0_done` the first-digit counts are already there: the approximate kernel left one

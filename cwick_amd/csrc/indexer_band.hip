@@ -30,9 +30,9 @@
 //      candidates by exact score, ties to the smaller index: one workgroup per row ranks the
 //      candidates and an ordered pass writes the indices (topk.hip).
 // Whenever a row does not fit this (more candidates than the list holds, a bound that is not
-// finite, NaN where T should be), the exact kernel runs for that row after all: it is always
-// launched and returns at once for rows that went well.
-#include "common.hpp"
+// finite, NaN where T should be), the rescoring kernel's workgroups run the exact kernel's code
+// on all keys of that row and the pick kernel's workgroup the plain select.
+#include "indexer_exact.hpp"
 
 namespace cwick {
 
@@ -257,7 +257,15 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
     __shared__ float terms[16][65];
     const int b = blockIdx.y, tid = threadIdx.x;
     const IndexerBandRow st = rows[b];
-    if (indexer_band_failed(st, cap)) return;
+    if (indexer_band_failed(st, cap)) {
+        // the row did not fit the band: the workgroups of this launch score all of its keys
+        // with the exact kernel's code instead
+        for (int64_t block = blockIdx.x; block * IDX_THREADS < n_keys; block += gridDim.x) {
+            indexer_exact_block(keys, kscale, key_bstride, kscale_bstride, n_keys, q, w, ih, scores, b, block);
+            __syncthreads();
+        }
+        return;
+    }
     const int c0 = blockIdx.x * 16;
     if (c0 >= (int)st.n_cand) return;
     const int j = tid & 15, hg = tid >> 4;                          // candidate, head group
@@ -386,10 +394,6 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
         keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores, cand_score);
     CWICK_HIP_CALL(hipGetLastError());
-    // rows that did not fit the band take the exact kernel after all
-    if (!launch_indexer_scores_rows(keys, kscale, key_bstride, kscale_bstride, batch, n_keys, q_idx, w,
-                                    n_idx_heads, scores, rows, cap, s))
-        return 0;
     }
     return launch_topk_band_finish(scores, batch, n_keys, k, cand, cand_score, cap, rows, hi_count, out_idx, s);
 }
