@@ -37,12 +37,13 @@
 namespace cwick {
 
 constexpr int IB_THREADS = 256;
+constexpr int IB_QROW = 128 + 8;                 // bf16 per head row of q in LDS (padded: 272 bytes)
 constexpr int IB_KEYS = CWICK_INDEXER_APPROX_KEYS;   // keys per workgroup of the approximate kernel
 constexpr int IB_HD = CWICK_HIP_INDEX_DIM;    // 128
 
 typedef __attribute__((ext_vector_type(2))) float ib_f32x2;
 
-__global__ void __launch_bounds__(IB_THREADS)
+__global__ void __launch_bounds__(IB_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict__ kscale,
                       int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
                       const uint16_t *__restrict__ q,   // [batch][ih][128] bf16
@@ -52,6 +53,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       uint32_t *__restrict__ digit0, size_t digit0_row) {   // optional: first-digit counts for the radix select
     __shared__ float c_sh[1][IB_HD];
     __shared__ uint32_t hist0[256 * 8];
+    __shared__ __attribute__((aligned(16))) uint16_t q_sh[64 * IB_QROW];
     __shared__ float w_sh[64];
     __shared__ float bmax_sh[IB_THREADS / 64];
     const int b = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
@@ -81,27 +83,39 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         for (int i = 0; i < 4; i++) raw[i] = *(const u32x4 *)(krow + 16 * i);
         kst = ksb[tc];
     };
-    // A operands (rows = heads).  Their loads go out first and the first two key iterations
-    // right behind them: loads return in order, so the bound row below is worked out of the
-    // operand registers while the keys are still on their way
+    // A operands (rows = heads): every wave needs all of q, so the workgroup fetches it once
+    // (sixteen bytes per thread and step) and the waves take their fragments from LDS; rows are
+    // 272 bytes apart there, which spreads the sixteen-byte reads of consecutive heads over the
+    // banks.  The loads go out first and the first two key iterations right behind them.
     bf16x8 qa[2][8], ca[8];
+    {
+        u32x4 stage[4];
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            const int head = mb * 32 + row;
+        for (int j = 0; j < 4; j++) {
+            const int c = tid + IB_THREADS * j, head = c >> 4, part = c & 15;
             const int hc = head < ih ? head : ih - 1;           // clamped load, zeroed afterwards
-            u32x4 v = *(const u32x4 *)(qb + (size_t)hc * IB_HD + 64 * g + 8 * ks);
-            if (head >= ih) v = (u32x4){0u, 0u, 0u, 0u};
-            qa[mb][ks] = __builtin_bit_cast(bf16x8, v);
+            stage[j] = *(const u32x4 *)(qb + (size_t)hc * IB_HD + 8 * part);
+            if (head >= ih) stage[j] = (u32x4){0u, 0u, 0u, 0u};
         }
+        load_keys(0, raw_a, kst_a);
+        load_keys(1, raw_b, kst_b);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int c = tid + IB_THREADS * j;
+            *(u32x4 *)&q_sh[(c >> 4) * IB_QROW + 8 * (c & 15)] = stage[j];
+        }
+    }
     if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) hist0[tid + IB_THREADS * j] = 0u;
     const float w0_abs = row < ih ? fabsf(wb[row]) : 0.0f;
     const float w1_abs = row + 32 < ih ? fabsf(wb[row + 32]) : 0.0f;
-    load_keys(0, raw_a, kst_a);
-    load_keys(1, raw_b, kst_b);
+    __syncthreads();
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++)
+            qa[mb][ks] = *(const bf16x8 *)&q_sh[(mb * 32 + row) * IB_QROW + 64 * g + 8 * ks];
     {   // c_i = sum_h |w_h| |q_hi| from the operand registers: lane (row, g) holds dims 64 g .. +63
         // of heads row and row + 32; a reduce-scatter over the 32 lanes of a half (exchange half
         // of the values, add, five times) leaves dims 64 g + 2 row + {0, 1} in each lane
