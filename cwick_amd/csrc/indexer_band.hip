@@ -51,7 +51,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
                       IndexerBandRow *__restrict__ rows,
                       uint32_t *__restrict__ digit0, size_t digit0_row) {   // optional: first-digit counts for the radix select
-    __shared__ float c_sh[1][IB_HD];
+    __shared__ float c_sh[2][IB_HD];
     __shared__ uint32_t hist0[256 * 8];
     __shared__ __attribute__((aligned(16))) uint16_t q_sh[64 * IB_QROW];
     __shared__ float w_sh[64];
@@ -108,43 +108,21 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) hist0[tid + IB_THREADS * j] = 0u;
-    const float w0_abs = row < ih ? fabsf(wb[row]) : 0.0f;
-    const float w1_abs = row + 32 < ih ? fabsf(wb[row + 32]) : 0.0f;
     __syncthreads();
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll
         for (int ks = 0; ks < 8; ks++)
             qa[mb][ks] = *(const bf16x8 *)&q_sh[(mb * 32 + row) * IB_QROW + 64 * g + 8 * ks];
-    {   // c_i = sum_h |w_h| |q_hi| from the operand registers: lane (row, g) holds dims 64 g .. +63
-        // of heads row and row + 32; a reduce-scatter over the 32 lanes of a half (exchange half
-        // of the values, add, five times) leaves dims 64 g + 2 row + {0, 1} in each lane
-        const float w0 = w0_abs, w1 = w1_abs;
-        float val[64];
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            const u32x4 x0 = __builtin_bit_cast(u32x4, qa[0][ks]), x1 = __builtin_bit_cast(u32x4, qa[1][ks]);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                val[8 * ks + 2 * j] = w0 * fabsf(bf16lo_to_f32(x0[j])) + w1 * fabsf(bf16lo_to_f32(x1[j]));
-                val[8 * ks + 2 * j + 1] = w0 * fabsf(bf16hi_to_f32(x0[j])) + w1 * fabsf(bf16hi_to_f32(x1[j]));
-            }
+    {   // c_i = sum_h |w_h| |q_hi|: thread (i, half) adds up 32 heads of dimension i out of LDS
+        const int i = tid & (IB_HD - 1), half = tid >> 7;
+        float c = 0.0f;
+#pragma unroll 8
+        for (int h = 0; h < 32; h++) {
+            const int head = 32 * half + h;
+            c = __builtin_fmaf(fabsf(w_sh[head]), fabsf(bf16_to_f32(q_sh[head * IB_QROW + i])), c);
         }
-#define CWICK_IB_RS(m, n)                                                                \
-    {                                                                                    \
-        const bool up = (lane & (m)) != 0;                                               \
-        _Pragma("unroll") for (int i = 0; i < (n); i++) {                                \
-            const float send = up ? val[i] : val[i + (n)];                               \
-            const float keep = up ? val[i + (n)] : val[i];                               \
-            val[i] = keep + __shfl_xor(send, (m), 64);                                   \
-        }                                                                                \
-    }
-        CWICK_IB_RS(16, 32) CWICK_IB_RS(8, 16) CWICK_IB_RS(4, 8) CWICK_IB_RS(2, 4) CWICK_IB_RS(1, 2)
-#undef CWICK_IB_RS
-        if (wave == 0) {
-            c_sh[0][64 * g + 2 * row] = val[0];
-            c_sh[0][64 * g + 2 * row + 1] = val[1];
-        }
+        c_sh[half][i] = c;
     }
     __syncthreads();
 #pragma unroll
@@ -155,8 +133,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
             for (int j = 0; j < 4; j++) {
                 // rounded up to bf16
                 const int i0 = 64 * g + 8 * ks + 2 * j;
-                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0]) + 0xFFFFu) >> 16;
-                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1]) + 0xFFFFu) >> 16;
+                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0] + c_sh[1][i0]) + 0xFFFFu) >> 16;
+                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1] + c_sh[1][i0 + 1]) + 0xFFFFu) >> 16;
                 v[j] = lo | (hi << 16);
             }
         }
