@@ -106,6 +106,7 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
 // The end of the banded select, after the candidates have their exact scores: ranks the
 // candidates, writes the selected indices of every row that fitted the band, and runs the
 // plain select for the rows that did not (their scores are the exact kernel's by then).
+// `scores` is only read.
 // hi_count: [batch][64] dwords, filled by launch_topk_band_classify.
 // cand_score: [batch][cap], the exact score of every list entry (what the rescoring wrote).
 int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand,

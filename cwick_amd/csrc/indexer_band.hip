@@ -27,11 +27,11 @@
 //   4. indexer_rescore_kernel: the reference's arithmetic, instruction for instruction as in
 //      indexer.hip, for the candidates only, spread over heads so that it takes microseconds.
 //   5. the selection is the +inf keys (fewer than k, all selected) and the best k - (their number)
-//      candidates by exact score, ties to the smaller index: one workgroup per row ranks the
-//      candidates and an ordered pass writes the indices (topk.hip).
+//      candidates by exact score, ties to the smaller index: topk_band_finish_kernel (topk.hip)
+//      ranks the candidates and writes the indices in order.
 // Whenever a row does not fit this (more candidates than the list holds, a bound that is not
 // finite, NaN where T should be), the rescoring kernel's workgroups run the exact kernel's code
-// on all keys of that row and the pick kernel's workgroup the plain select.
+// on all keys of that row and the finish kernel's first workgroup the plain select.
 #include "indexer_exact.hpp"
 
 namespace cwick {

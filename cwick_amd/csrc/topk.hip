@@ -625,11 +625,14 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
 // selected (+inf, hi_count[w] of them in workgroup w's stretch), keys that are certainly not
 // (-inf) and at most `cap` candidates with their exact scores.  The selection is the +inf keys
 // and the best need = k - (number of +inf keys) candidates, ties to the smaller index as
-// everywhere.  One workgroup per row ranks the candidates (a radix select on the order keys of
-// their scores, and, if the need-th key has ties that do not all fit, a second one on the
-// inverted indices of the tied), turns the chosen ones into +inf and the others into -inf and
-// adds them to hi_count; the emit kernel then only has to write out the +inf keys in index
-// order.
+// everywhere.  The workgroups of a row are those of the classify kernel (2048 keys each).  Every
+// one of them ranks the candidates for itself (a radix select on the order keys of their
+// scores, and, if the need-th key has ties that do not all fit, a second one on the inverted
+// indices of the tied): the list is at most 4096 entries, and knowing the outcome everywhere
+// saves a launch, the write-back of the decisions and the atomics that would count them.  A
+// workgroup then starts writing after the +inf keys of the stretches before it (hi_count) and
+// the chosen candidates among them (counted out of the list), and writes its own keys that
+// are +inf or chosen candidates in index order.
 constexpr int TOPK_BAND_THREADS = 1024;
 constexpr int TOPK_BAND_EPT = CWICK_INDEXER_BAND_CAP / TOPK_BAND_THREADS;     // 4
 
@@ -721,36 +724,46 @@ __device__ __forceinline__ void topk_band_select(const uint32_t (&val)[TOPK_BAND
 }
 
 __global__ void __launch_bounds__(TOPK_BAND_THREADS)
-topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
-                      const int32_t *__restrict__ cand, const float *__restrict__ cand_score, int cap,
-                      const IndexerBandRow *__restrict__ rows, uint32_t *__restrict__ hi_count,
-                      int32_t *__restrict__ out) {
+topk_band_finish_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int n_wg,
+                        const int32_t *__restrict__ cand, const float *__restrict__ cand_score, int cap,
+                        const IndexerBandRow *__restrict__ rows, const uint32_t *__restrict__ hi_count,
+                        int32_t *__restrict__ out) {
+    constexpr int KPT = TOPK_MW_KEYS / TOPK_BAND_THREADS;           // own keys per thread: 2
     __shared__ TopkBandShared sh;
-    __shared__ uint32_t sh_hi;
-    const int row = blockIdx.x, tid = threadIdx.x;
-    // the whole list is loaded whatever its length (the thread count times four is its
-    // capacity): these loads then travel together with the row state they would depend on
+    __shared__ uint32_t sh_hi, sh_before;
+    __shared__ uint32_t sh_cnt[KPT][TOPK_BAND_THREADS / 64];
+    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const float *sc = scores + (size_t)row * n;
+    int32_t *dst = out + (size_t)row * k;
+    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
+    // every load first, one round trip: the whole candidate list whatever its length (the
+    // thread count times four is its capacity), this stretch's scores, the counts, the row state
     int32_t idx[TOPK_BAND_EPT];
-    float val[TOPK_BAND_EPT];
+    float val[TOPK_BAND_EPT], v[KPT];
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++) {
         idx[j] = cand[(size_t)row * cap + tid + TOPK_BAND_THREADS * j];
         val[j] = cand_score[(size_t)row * cap + tid + TOPK_BAND_THREADS * j];
     }
-    uint32_t *hc = hi_count + (size_t)row * TOPK_MW_MAX_WGS;
-    const uint32_t hi_part = tid < n_wg ? hc[tid] : 0u;
+#pragma unroll
+    for (int j = 0; j < KPT; j++) {
+        const int64_t i = base + j * TOPK_BAND_THREADS + tid;
+        v[j] = sc[i < n ? i : n - 1];
+    }
+    const uint32_t hi_part = tid < n_wg ? hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid] : 0u;
     const IndexerBandRow st = rows[row];
-    float *sc = scores + (size_t)row * n;
     if (indexer_band_failed(st, cap)) {
-        // the row did not fit the band: its scores are the exact kernel's by now, and this
-        // workgroup selects from all of them (the emit kernel skips the row)
-        topk_radix_row(sc, n, k, out + (size_t)row * k);
+        // the row did not fit the band: its scores are the exact kernel's by now, and its first
+        // workgroup selects from all of them
+        if (wg == 0) topk_radix_row(sc, n, k, dst);
         return;
     }
     const int n_cand = (int)st.n_cand;
-    if (tid == 0) sh_hi = 0u;
+    if (tid == 0) sh_hi = 0u, sh_before = 0u;
     __syncthreads();
     if (tid < n_wg) atomicAdd(&sh_hi, hi_part);
+    if (tid < wg) atomicAdd(&sh_before, hi_part);
     uint32_t key[TOPK_BAND_EPT], inv[TOPK_BAND_EPT], live = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++) {
@@ -772,63 +785,39 @@ topk_band_pick_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_wg
             topk_band_select(inv, tied, r, sh, T2, r2, e2);
         }
     }
+    // a candidate is chosen if it is above the need-th, or ties with it and has a small enough index
+    auto chosen = [&](uint32_t kk, uint32_t ii) { return need > 0u && (kk > T || (kk == T && ii >= T2)); };
+    // chosen candidates in the stretches before this one
+    uint32_t earlier = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++)
-        if (live >> j & 1u) {
-            const bool take = need > 0u && (key[j] > T || (key[j] == T && inv[j] >= T2));
-            sc[idx[j]] = take ? INFINITY : -INFINITY;
-            if (take) atomicAdd(&hc[idx[j] / TOPK_MW_KEYS], 1u);
-        }
-}
-
-// writes the indices of a row's +inf keys in ascending order; workgroup w starts after the
-// hi_count of the workgroups before it
-__global__ void __launch_bounds__(TOPK_MW_THREADS)
-topk_band_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
-                      const IndexerBandRow *__restrict__ rows, int cap,
-                      const uint32_t *__restrict__ hi_count, int32_t *__restrict__ out) {
-    __shared__ uint32_t sh_before;
-    __shared__ uint32_t sh_cnt[TOPK_MW_EPT][TOPK_MW_THREADS / 64];
-    const int row = blockIdx.y, wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const float *sc = scores + (size_t)row * n;
-    int32_t *dst = out + (size_t)row * k;
-    const int64_t base = (int64_t)wg * TOPK_MW_KEYS;
-    float v[TOPK_MW_EPT];                       // all loads first: one round trip
+        if ((live >> j & 1u) && (int64_t)idx[j] < base && chosen(key[j], inv[j])) earlier++;
+    if (earlier) atomicAdd(&sh_before, earlier);
+    // own keys: +inf is in, -inf is out, anything else is a candidate with its exact score.
+    // Element (j, tid) is index base + 1024 j + tid: the order of the workgroup is (j, wave, lane)
+    uint64_t m[KPT];
 #pragma unroll
-    for (int j = 0; j < TOPK_MW_EPT; j++) {
-        const int64_t i = base + j * TOPK_MW_THREADS + tid;
-        const int64_t ic = i < n ? i : n - 1;
-        v[j] = sc[ic];
-        if (i >= n) v[j] = 0.0f;
-    }
-    const uint32_t before_part = tid < wg ? hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid] : 0u;
-    if (indexer_band_failed(rows[row], cap)) return;
-    if (tid == 0) sh_before = 0u;
-    __syncthreads();
-    if (tid < wg) atomicAdd(&sh_before, before_part);
-    // element (j, tid) is index base + 256 j + tid: the order of the workgroup is (j, wave, lane)
-    uint64_t m[TOPK_MW_EPT];
-#pragma unroll
-    for (int j = 0; j < TOPK_MW_EPT; j++) {
-        m[j] = __ballot(v[j] == INFINITY);
+    for (int j = 0; j < KPT; j++) {
+        const int64_t i = base + j * TOPK_BAND_THREADS + tid;
+        const bool in = i < n && (v[j] == INFINITY || (v[j] != -INFINITY && chosen(topk_key(v[j]), ~(uint32_t)i)));
+        m[j] = __ballot(in);
         if (lane == 0) sh_cnt[j][wave] = (uint32_t)__builtin_popcountll(m[j]);
     }
     __syncthreads();
-    uint32_t run = sh_before, my_pos[TOPK_MW_EPT];
+    uint32_t run = sh_before, my_pos[KPT];
 #pragma unroll
-    for (int j = 0; j < TOPK_MW_EPT; j++)
+    for (int j = 0; j < KPT; j++)
 #pragma unroll
-        for (int w = 0; w < TOPK_MW_THREADS / 64; w++) {
+        for (int w = 0; w < TOPK_BAND_THREADS / 64; w++) {
             if (w == wave) my_pos[j] = run;
             run += sh_cnt[j][w];
         }
     const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
 #pragma unroll
-    for (int j = 0; j < TOPK_MW_EPT; j++)
+    for (int j = 0; j < KPT; j++)
         if ((m[j] >> lane) & 1) {
             const uint32_t pos = my_pos[j] + (uint32_t)__builtin_popcountll(m[j] & lt);
-            if (pos < (uint32_t)k) dst[pos] = (int32_t)(base + j * TOPK_MW_THREADS + tid);
+            if (pos < (uint32_t)k) dst[pos] = (int32_t)(base + j * TOPK_BAND_THREADS + tid);
         }
 }
 
@@ -870,15 +859,15 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
 int launch_topk_band_finish(float *scores, int batch, int64_t n, int64_t k, const int32_t *cand,
                             const float *cand_score, int cap, const IndexerBandRow *rows, uint32_t *hi_count,
                             int32_t *out_idx, hipStream_t s) {
-    static_assert(TOPK_BAND_EPT * TOPK_BAND_THREADS == CWICK_INDEXER_BAND_CAP, "the pick kernel holds the whole list");
-    static_assert(TOPK_BAND_THREADS == TOPK_THREADS, "the pick kernel runs the one-workgroup select for rows off the band");
+    static_assert(TOPK_BAND_EPT * TOPK_BAND_THREADS == CWICK_INDEXER_BAND_CAP, "a workgroup holds the whole list");
+    static_assert(TOPK_BAND_THREADS == TOPK_THREADS, "the workgroup runs the one-workgroup select for rows off the band");
+    static_assert(TOPK_MW_KEYS % TOPK_BAND_THREADS == 0, "whole keys per thread");
     const int64_t n_wg = topk_mw_wgs(n);
     CWICK_REQUIRE(n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS && cap == CWICK_INDEXER_BAND_CAP && k < n,
                   "topk_band_finish: n %lld out of range", (long long)n);
     ProfScope ps(CWICK_HIP_PROF_TOPK, s);
-    topk_band_pick_kernel<<<batch, TOPK_BAND_THREADS, 0, s>>>(scores, n, k, (int)n_wg, cand, cand_score, cap, rows, hi_count, out_idx);
-    topk_band_emit_kernel<<<dim3((unsigned)n_wg, (unsigned)batch), TOPK_MW_THREADS, 0, s>>>(scores, n, k, rows, cap,
-                                                                                              hi_count, out_idx);
+    topk_band_finish_kernel<<<dim3((unsigned)n_wg, (unsigned)batch), TOPK_BAND_THREADS, 0, s>>>(
+        scores, n, k, (int)n_wg, cand, cand_score, cap, rows, hi_count, out_idx);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }
