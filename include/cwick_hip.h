@@ -242,6 +242,11 @@ int cwick_hip_indexer_scores_dev(const uint8_t *keys, const float *kscale,
 int cwick_hip_topk_dev(const float *scores, int batch, int64_t n, int64_t k,
                        int32_t *out_idx, void *stream);
 
+/* The fused step of cwick_hip_dsa_decode on device operands.  scores_tmp
+ * [batch][n_keys] floats is scratch: what it holds afterwards are not the
+ * indexer's scores (the fused select overwrites most of them with +inf / -inf
+ * marks); cwick_hip_indexer_scores_dev returns scores.  sel_out [batch][topk]
+ * receives the selected rows and is required. */
 int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale,
                              int64_t key_batch_stride, int64_t kscale_batch_stride,
                              const uint8_t *rows, const float *scales,
