@@ -153,7 +153,10 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         const int64_t t = wbase + it * 32 + row;
         const bool live = t < n_keys;
         // the accumulators are pinned to VGPRs (through the builtin they land in AGPRs and cost a
-        // read each); the compiler does not see these as MFMAs, hence the wait before the reads
+        // read each); the compiler does not see these as MFMAs and leaves out the wait states
+        // they need: two between a VALU write of an operand and the MFMA that reads it (the
+        // s_nop 1 in front of the first MFMA after the conversions and of the one after the
+        // masks), and the wait before the results are read
         f32x16 d0, d1, ab;
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
@@ -169,21 +172,30 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
 #pragma unroll
             for (int j = 0; j < 4; j++) ea[j] = e[j] & 0x7FFF7FFFu;
             if (ks == 0) {
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d0) : "v"(qa[0][ks]), "v"(e));
+                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d0) : "v"(qa[0][ks]), "v"(e));
                 asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d1) : "v"(qa[1][ks]), "v"(e));
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(ab) : "v"(ca[ks]), "v"(ea));
+                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(ab) : "v"(ca[ks]), "v"(ea));
             } else {
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d0) : "v"(qa[0][ks]), "v"(e));
+                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d0) : "v"(qa[0][ks]), "v"(e));
                 asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d1) : "v"(qa[1][ks]), "v"(e));
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ab) : "v"(ca[ks]), "v"(ea));
+                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ab) : "v"(ca[ks]), "v"(ea));
             }
         }
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        // Nothing may write a register that these MFMAs read before they are done (they read
+        // their operands pass by pass, and the compiler does not know them as MFMAs): the
+        // instructions that follow the last one wait, and carry the accumulators, so that
+        // nothing that reads those can be scheduled above the wait either.
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d0), "+v"(d1), "+v"(ab)::"memory");
         float sp = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            sp = __builtin_fmaf(wl[0][i], __builtin_amdgcn_fmed3f(d0[i], 0.0f, INFINITY), sp);
-            sp = __builtin_fmaf(wl[1][i], __builtin_amdgcn_fmed3f(d1[i], 0.0f, INFINITY), sp);
+            // one instruction per ReLU (through fmaxf or fmed3 the compiler adds a second one
+            // that quiets NaNs; a NaN dot counts as 0 here, and the bound row turns NaN with it)
+            float r0, r1;
+            asm("v_max_f32 %0, 0, %1" : "=v"(r0) : "v"(d0[i]));
+            asm("v_max_f32 %0, 0, %1" : "=v"(r1) : "v"(d1[i]));
+            sp = __builtin_fmaf(wl[0][i], r0, sp);
+            sp = __builtin_fmaf(wl[1][i], r1, sp);
         }
         sp += __shfl_xor(sp, 32, 64);
         const float band = ab[0] + __shfl_xor(ab[0], 32, 64);      // row 0 sits in the g = 0 lanes
