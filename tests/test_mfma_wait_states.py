@@ -1,0 +1,56 @@
+"""The kernels that issue matrix instructions from inline assembly (to pin their accumulators to
+VGPRs) hide them from the compiler's hazard recognizer, which would otherwise put two wait states
+between a vector-ALU write of a register and the MFMA that reads it as an operand.  The sources
+place `s_nop 1` where such a write comes last; this test compiles them to assembly and checks the
+rule on what the compiler scheduled: no vector-ALU instruction that writes an MFMA's A or B operand
+may be one of the two instructions in front of it.  (Violations give wrong numbers only now and
+then, depending on timing, which is why the rule is checked on the code and not on results.)"""
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+
+from cwick_amd import build as B
+
+ASM_MFMA_SOURCES = ["gqa_prefill.hip", "indexer_band.hip"]
+
+
+def _regs(tok):
+    m = re.match(r"v\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"v(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
+
+
+@pytest.mark.parametrize("src", ASM_MFMA_SOURCES)
+def test_no_valu_write_right_before_an_mfma_reads_it(src):
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        cmd = [B._hipcc()] + B.COMMON + B.PER_FILE.get(src, []) + [
+            "-w", "-S", "--cuda-device-only", os.path.join(B.CSRC, src), "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        ins = []
+        for line in open(out):
+            t = line.strip()
+            if not t or t.startswith((";", ".")) or t.endswith(":"):
+                continue
+            ins.append(t)
+    n_mfma, bad = 0, []
+    for i, t in enumerate(ins):
+        if not t.startswith("v_mfma"):
+            continue
+        n_mfma += 1
+        ops = [o.strip() for o in t.split(None, 1)[1].split(",")]
+        src_regs = _regs(ops[1]) | _regs(ops[2])
+        for back in (1, 2):
+            p = ins[i - back]
+            if p.startswith("v_") and not p.startswith("v_mfma"):
+                dst = _regs(p.split(None, 1)[1].split(",")[0].strip())
+                if dst & src_regs:
+                    bad.append((p, t))
+    assert n_mfma > 0
+    assert not bad, "VALU write within two instructions of the MFMA that reads it: %r" % bad[:3]
