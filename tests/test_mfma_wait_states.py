@@ -3,7 +3,8 @@ VGPRs) hide them from the compiler's hazard recognizer, which would otherwise pu
 between a vector-ALU write of a register and the MFMA that reads it as an operand.  The sources
 place `s_nop 1` where such a write comes last; this test compiles them to assembly and checks the
 rule on what the compiler scheduled: no vector-ALU instruction that writes an MFMA's A or B operand
-may be one of the two instructions in front of it.  (Violations give wrong numbers only now and
+may be one of the two instructions in front of it, and no instruction may read an MFMA's result
+within nineteen wait states of it unless it is an MFMA accumulating into it.  (Violations give wrong numbers only now and
 then, depending on timing, which is why the rule is checked on the code and not on results.)"""
 import os
 import re
@@ -39,7 +40,7 @@ def test_no_valu_write_right_before_an_mfma_reads_it(src):
             if not t or t.startswith((";", ".")) or t.endswith(":"):
                 continue
             ins.append(t)
-    n_mfma, bad = 0, []
+    n_mfma, bad, early = 0, [], []
     for i, t in enumerate(ins):
         if not t.startswith("v_mfma"):
             continue
@@ -52,5 +53,26 @@ def test_no_valu_write_right_before_an_mfma_reads_it(src):
                 dst = _regs(p.split(None, 1)[1].split(",")[0].strip())
                 if dst & src_regs:
                     bad.append((p, t))
+        # The other direction: a result must not be read by anything but an MFMA that accumulates
+        # into it before the matrix pipe has written it.  The compiler's own figure for the
+        # longest MFMA is 19 wait states (an s_nop N counts N + 1, any other instruction 1);
+        # the scan follows straight-line code and stops at a branch or after 24.
+        dst_regs = _regs(ops[0])
+        waited = 0
+        for q in ins[i + 1:i + 64]:
+            if q.startswith(("s_cbranch", "s_branch", "s_endpgm")) or waited >= 24:
+                break
+            qops = [o.strip() for o in q.split(None, 1)[1].split(",")] if " " in q else []
+            reads = set()
+            for o in (qops[1:] if q.startswith("v_") and not q.startswith("v_mfma") else qops):
+                reads |= _regs(o.split()[0]) if o else set()
+            if q.startswith("v_mfma"):
+                reads = _regs(qops[1]) | _regs(qops[2])          # accumulating into the result is allowed
+            if reads & dst_regs and waited < 19:
+                early.append((t[:60], q[:60], waited))
+                break
+            m = re.match(r"s_nop (\d+)", q)
+            waited += int(m.group(1)) + 1 if m else 1
     assert n_mfma > 0
     assert not bad, "VALU write within two instructions of the MFMA that reads it: %r" % bad[:3]
+    assert not early, "MFMA result read before the matrix pipe has written it: %r" % early[:3]
