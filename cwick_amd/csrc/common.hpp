@@ -34,9 +34,6 @@ int num_cus();
 // asks for more bytes; kernels enqueued earlier on the stream have finished
 // with it by the time a later enqueue on the same stream touches it.
 void *workspace(hipStream_t s, size_t bytes);
-// A second, independent scratch area on the same stream (staging of host
-// operands by the host-pointer entry points).
-void *staging(hipStream_t s, size_t bytes);
 
 // Phase timer: brackets the launches made while it is alive with two events on
 // `s` when profiling is enabled; does nothing (and records nothing) otherwise.
@@ -57,12 +54,13 @@ int launch_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64
                        float scale, float *out, hipStream_t s);
 int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
-                      const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
+                      const uint16_t *q, int n_heads, float scale, const float *sink, float *out,
+                      hipStream_t s);
 int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
                        const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
 int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys,
-                          const uint16_t *q_idx, const float *w, int n_idx_heads,
+                          const uint16_t *q_idx, const float *w, int n_idx_heads, int mode,
                           float *scores, hipStream_t s);
 // ---- fused select: approximate scores with an error band, exact scores for the keys inside it
 // (indexer_band.hip).  One of these per batch row, in the workspace:
@@ -119,6 +117,7 @@ int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *
 int launch_quant_ikeys(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,
                        hipStream_t s);
 int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s);
+int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
 
 // ---- device helpers ---------------------------------------------------------

@@ -49,6 +49,8 @@
 //   64-byte segments that fall into different banks.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace cwick {
 
 constexpr int PF_THREADS = 256;
@@ -690,12 +692,11 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
 
 // rows that see at most this many keys take the two-term-weight variant
 static int64_t gqa_precise_keys() {
-    static int64_t v = -1;
-    if (v < 0) {
+    static const int64_t v = [] {
         const char *e = getenv("CWICK_HIP_GQA_PRECISE_KEYS");
-        v = e ? atoll(e) : 1024;
-        if (v < 0) v = 0;
-    }
+        const int64_t x = e ? atoll(e) : 1024;
+        return x < 0 ? (int64_t)0 : x;
+    }();
     return v;
 }
 
@@ -703,13 +704,14 @@ template <int GROUP>
 static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
                            int n_kv_heads, const uint16_t *q, float scale, float *out,
                            hipStream_t s) {
-    static bool attr_set = false;
+    static std::once_flag attr_once;
+    static hipError_t attr_err = hipSuccess;
     const size_t smem = sizeof(PfSmem);
-    if (!attr_set) {
-        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    std::call_once(attr_once, [&] {
+        attr_err = hipFuncSetAttribute((const void *)gqa_prefill_kernel<GROUP>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    });
+    CWICK_HIP_CALL(attr_err);
     constexpr int P = PF_ROWS / GROUP;
     const int64_t pblocks = (n + P - 1) / P;
     CWICK_REQUIRE(pblocks * n_kv_heads <= 0x7FFFFFFF, "gqa_prefill: grid too large");

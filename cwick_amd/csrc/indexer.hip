@@ -42,23 +42,96 @@ indexer_scores_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     indexer_exact_block(keys, kscale, key_bstride, kscale_bstride, n_keys, q, w, ih, scores, blockIdx.y, blockIdx.x);
 }
 
+// The DeepSeek flavour of the same loop (ds_indexer, src/ds_model.c:1099-1121), bit for bit:
+//
+//     kt[i] = e4m3(key[t][i]) * kscale[t]          the dequantised key the reference holds in fp32
+//     d     = 0;  d = d + (q_h[i] * kt[i])         i = 0..127 in order, multiply and add rounded
+//                                                  separately (the product of an 8-bit and a
+//                                                  24-bit significand is not exact: no fma)
+//     d     = bf16_round(d)                        round-to-nearest-even onto the bf16 grid
+//     s     = s + d * bf16_round(w[h])  if d > 0   multiply, then add
+//
+// One key per lane, its 128 dequantised values in registers; q is widened to fp32 in LDS and
+// every lane reads the same address (a broadcast).  Twice the vector-ALU work of the kernel
+// above and one dependent chain per head: this is the mode for checking against that CPU path,
+// not the fast one.
+__global__ void __launch_bounds__(IDX_THREADS)
+indexer_scores_ds_kernel(const uint8_t *__restrict__ keys, const float *__restrict__ kscale,
+                         int64_t key_bstride, int64_t kscale_bstride, int64_t n_keys,
+                         const uint16_t *__restrict__ q, const float *__restrict__ w, int ih,
+                         float *__restrict__ scores) {
+    __shared__ __attribute__((aligned(16))) float qs[64 * IDX_HD];
+    __shared__ float ws[64];
+    const int b = blockIdx.y;
+    const int64_t t = (int64_t)blockIdx.x * IDX_THREADS + threadIdx.x;
+    const bool live = t < n_keys;
+    const int64_t tc = live ? t : n_keys - 1;
+    const uint8_t *krow = keys + (size_t)b * key_bstride + (size_t)tc * IDX_HD;
+    const float ks = kscale[(size_t)b * kscale_bstride + tc];
+    const uint16_t *qb = q + (size_t)b * ih * IDX_HD;
+    for (int i = threadIdx.x; i < ih * IDX_HD; i += IDX_THREADS) qs[i] = bf16_to_f32(qb[i]);
+    if ((int)threadIdx.x < ih)
+        ws[threadIdx.x] = __builtin_bit_cast(float, f32_to_bf16_rne(w[(size_t)b * ih + threadIdx.x]) << 16);
+    float e[IDX_HD];
+#pragma unroll
+    for (int c = 0; c < IDX_HD / 16; c++) {
+        const u32x4 v = *(const u32x4 *)(krow + c * 16);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const f32x2 lo = e4m3x2_to_f32<false>(v[j]);
+            const f32x2 hi = e4m3x2_to_f32<true>(v[j]);
+            e[c * 16 + j * 4 + 0] = lo[0] * ks;
+            e[c * 16 + j * 4 + 1] = lo[1] * ks;
+            e[c * 16 + j * 4 + 2] = hi[0] * ks;
+            e[c * 16 + j * 4 + 3] = hi[1] * ks;
+        }
+    }
+    __syncthreads();
+    float s = 0.0f;
+    for (int h = 0; h < ih; h++) {
+        const f32x4 *qh = (const f32x4 *)(qs + h * IDX_HD);
+        float d = 0.0f;
+#pragma unroll
+        for (int c = 0; c < IDX_HD / 4; c++) {
+            const f32x4 qv = qh[c];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float prod = qv[j] * e[4 * c + j];
+                d = d + prod;
+            }
+        }
+        d = __builtin_bit_cast(float, f32_to_bf16_rne(d) << 16);
+        if (d > 0.0f) {
+            const float prod = d * ws[h];
+            s = s + prod;
+        }
+    }
+    if (live) scores[(size_t)b * n_keys + t] = s;
+}
+
 int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_bstride,
                           int64_t kscale_bstride, int batch, int64_t n_keys,
-                          const uint16_t *q_idx, const float *w, int n_idx_heads, float *scores,
-                          hipStream_t s) {
+                          const uint16_t *q_idx, const float *w, int n_idx_heads, int mode,
+                          float *scores, hipStream_t s) {
     CWICK_REQUIRE(keys && kscale && q_idx && w && scores, "indexer_scores: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 65535, "indexer_scores: batch %d", batch);
     CWICK_REQUIRE(n_keys >= 1 && n_keys <= ((int64_t)1 << 30), "indexer_scores: n_keys %lld",
                   (long long)n_keys);
     CWICK_REQUIRE(n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_scores: n_idx_heads %d (1..64)",
                   n_idx_heads);
+    CWICK_REQUIRE(mode == CWICK_HIP_INDEXER_GLM || mode == CWICK_HIP_INDEXER_DS,
+                  "indexer_scores: unknown mode %d", mode);
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
                   "indexer_scores: keys and q must be 16-byte aligned");
     dim3 grid((unsigned)((n_keys + IDX_THREADS - 1) / IDX_THREADS), batch);
     {
         ProfScope ps(CWICK_HIP_PROF_INDEXER, s);
-        indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
-                                                           n_keys, q_idx, w, n_idx_heads, scores);
+        if (mode == CWICK_HIP_INDEXER_DS)
+            indexer_scores_ds_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
+                                                                  n_keys, q_idx, w, n_idx_heads, scores);
+        else
+            indexer_scores_kernel<<<grid, IDX_THREADS, 0, s>>>(keys, kscale, key_bstride, kscale_bstride,
+                                                               n_keys, q_idx, w, n_idx_heads, scores);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

@@ -68,6 +68,14 @@ __global__ void __launch_bounds__(256) narrow_bf16_kernel(const float *__restric
     for (; i < n; i += stride) dst[i] = (uint16_t)f32_to_bf16_rne(src[i]);
 }
 
+// bf16 rows back to fp32 (q35_widen_rows, src/q35_model.c:1543-1556): exact
+__global__ void __launch_bounds__(256) widen_bf16_kernel(const uint16_t *__restrict__ src, int64_t n,
+                                                         float *__restrict__ dst) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < n; i += stride) dst[i] = bf16_to_f32(src[i]);
+}
+
 __global__ void __launch_bounds__(256) e4m3_table_kernel(float *out) {
     const uint32_t b = threadIdx.x;
     // the byte in the low and in the high half of the word must decode alike
@@ -111,6 +119,15 @@ int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s
     int64_t blocks = (n + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     narrow_bf16_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(src, n, dst);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s) {
+    CWICK_REQUIRE(src && dst && n > 0, "widen_bf16: bad argument");
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    widen_bf16_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(src, n, dst);
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -41,6 +41,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace cwick {
 namespace {
@@ -83,9 +84,17 @@ struct Params {
     float scale;
     int n_splits;
     int64_t keys_per_split;   // multiple of TK
+    const float *sink;        // per head, natural-log units of the scaled scores, or null
     float *out, *part_ml;
     uint32_t *part_acc;
 };
+
+// What a masked position of a tile (past the end of the list, a -1 or out-of-range entry of
+// sel[]) is fetched from: a row of zero bytes with zero scales.  Its weight is zero already;
+// with zero values and zero scales nothing of any cache row that is not in the list (a NaN
+// byte, a scale many binades above the others) can reach the products or the fp16 normaliser.
+__device__ __attribute__((aligned(16))) uint8_t g_zero_row[KDIM + 64] = {0};
+__device__ __attribute__((aligned(16))) float g_zero_scales[8] = {0.0f};
 
 struct Tile {
     uint8_t kv[NCOL][TK][16];     // [16-byte column][key][16]     36864 B
@@ -171,7 +180,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         return (int)r;
     };
     // global -> LDS copies in assembly: the compiler keeps no account of them, so nothing in the
-    // loop waits for the tile in flight except the s_waitcnt before the barrier
+    // loop waits for the tile in flight except the s_waitcnt before the barrier.  Each statement
+    // writes M0 itself right before the copy that reads it.  M0 is a reserved register to the
+    // compiler (it cannot be named as clobbered); what keeps this safe is that nothing else in
+    // this file makes the compiler use M0, which tests/test_mfma_wait_states.py checks on the
+    // compiled code.
     auto dma16 = [&](const void *gp, const void *lp) {
         const uint32_t off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void *)lp);
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gp), "s"(off) : "memory");
@@ -182,18 +195,19 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     };
     // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; wave w copies pieces w, w+12, w+24, w+36
     auto issue = [&](int r, Tile *b) {
-        const int64_t rc = r >= 0 ? r : 0;            // masked positions fetch row 0, weight 0
-        const uint8_t *gsrc = rows + rc * KDIM + 16 * wave;
+        // masked positions fetch the zero row
+        const uint8_t *gsrc = (r >= 0 ? rows + (int64_t)r * KDIM : g_zero_row) + 16 * wave;
         dma16(gsrc, &b->kv[wave][0][0]);
         dma16(gsrc + 192, &b->kv[wave + 12][0][0]);
         dma16(gsrc + 384, &b->kv[wave + 24][0][0]);
-        if (wave < 5) dma4(scales + rc * NBLK + wave, &b->sc[wave][0]);
+        if (wave < 5) dma4((r >= 0 ? scales + (int64_t)r * NBLK : g_zero_scales) + wave, &b->sc[wave][0]);
     };
 
     // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks
-    auto piece = [&](int pc, int64_t rc, Tile *b) {
-        if (pc < NCOL) dma16(rows + rc * KDIM + 16 * pc, &b->kv[pc][0][0]);
-        else if (pc < NCOL + NBLK) dma4(scales + rc * NBLK + (pc - NCOL), &b->sc[pc - NCOL][0]);
+    auto piece = [&](int pc, int r, Tile *b) {
+        if (pc < NCOL) dma16((r >= 0 ? rows + (int64_t)r * KDIM : g_zero_row) + 16 * pc, &b->kv[pc][0][0]);
+        else if (pc < NCOL + NBLK)
+            dma4((r >= 0 ? scales + (int64_t)r * NBLK : g_zero_scales) + (pc - NCOL), &b->sc[pc - NCOL][0]);
     };
     // Only tile 0 is fetched before the loop, by everybody.  In step -1, while tile 0 is scored,
     // the value waves (nothing to accumulate yet) fetch tile 1, and the scoring waves fetch tile 2
@@ -297,7 +311,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             const int row_now = row_nxt;              // rows of tile t+1, fetched one step ahead
             row_nxt = row_of(t + 2);
             const bool do_copy = t + 3 < n_tiles;
-            const int row_cp = do_copy ? row_of(t + 3) : 0;
+            const int row_cp = do_copy ? row_of(t + 3) : -1;
             if (t >= 0) {
                 // what the four key blocks of tile t used as reference for this half's heads
                 const f32x4 ml = *(const f32x4 *)&sm.x[t & 1].m[hh][n][0];
@@ -385,7 +399,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             // share of tile t+3 goes out now, when the wave would otherwise wait at the barrier
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (do_copy) {
-                const int64_t rc = row_cp >= 0 ? row_cp : 0;
+                const int rc = row_cp;
                 if (t >= 0) {
 #pragma unroll
                     for (int i = 0; i < (NCOL + NBLK - 4 * NV + 7) / 8; i++) piece(4 * NV + wave + 8 * i, rc, &sm.tile[(t + 3) % NST]);
@@ -418,9 +432,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         // waves copy (the scoring waves are the long pole of a step, and a wave that issues copies
         // stalls while the memory pipeline takes them): wave cw takes pieces cw, cw + 4, ...
         auto issue_value = [&](int r, Tile *b) {
-            const int64_t rc = r >= 0 ? r : 0;            // masked positions fetch row 0, weight 0
 #pragma unroll
-            for (int i = 0; i < NV; i++) piece(cw + 4 * i, rc, b);
+            for (int i = 0; i < NV; i++) piece(cw + 4 * i, r, b);
         };
         asm volatile("" ::: "memory");
 #pragma clang loop unroll(disable)
@@ -429,9 +442,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             if (do_copy) issue_value(row_of(t + 3), &sm.tile[(t + 3) % NST]);   // the stage tile t-1 left at the last barrier
             if (t < 0 && n_tiles > 1) {                   // all of tile 1
                 const int r = row_of(1);
-                const int64_t rc = r >= 0 ? r : 0;
 #pragma unroll
-                for (int i = 0; i < (NCOL + NBLK + 3) / 4; i++) piece(cw + 4 * i, rc, &sm.tile[1]);
+                for (int i = 0; i < (NCOL + NBLK + 3) / 4; i++) piece(cw + 4 * i, r, &sm.tile[1]);
             }
             if (t >= 0) {
                 // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 32 heads, tile t ----
@@ -545,9 +557,13 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 #pragma unroll
         for (int h2 = 0; h2 < 2; h2++) {
             const f32x4 lv = *(const f32x4 *)&lsum[(h2 * 16 + n) * 4];
-            const float L = (lv[0] + lv[1]) + (lv[2] + lv[3]);
+            float L = (lv[0] + lv[1]) + (lv[2] + lv[3]);
             const int head = hb * HW + 16 * h2 + n;
             if (head >= p.nh) continue;
+            // the attention sink of src/ds_model.c:946: one more term in the denominator, no value
+            // (with several splits the merge kernel adds it)
+            if (p.sink && p.n_splits == 1 && m_ref[h2] > -INFINITY)
+                L += __builtin_amdgcn_exp2f(p.sink[head] * 1.44269504088896340736f - m_ref[h2]);
             const float unit_f = e_run == E_NONE ? 0.0f : pow2i(e_run - WEXP);   // the accumulators are in units of 2^(e_run - WEXP)
             const float fin = p.n_splits == 1 ? (L > 0.0f ? unit_f / L : 0.0f) : unit_f;
             const size_t pb = ((size_t)y * p.n_splits + split) * (2 * n_hb) + 2 * hb + h2;
@@ -614,7 +630,8 @@ __device__ __forceinline__ void merge_add(f32x4 &acc, float &ls, const u32x2 a, 
 }
 __global__ void __launch_bounds__(64 * MW)
 mla_merge_frag16_kernel(const uint32_t *__restrict__ part_acc, const float *__restrict__ part_ml,
-                        int n_splits, int n_hb16, int nh, float *__restrict__ out, int packed) {
+                        int n_splits, int n_hb16, int nh, const float *__restrict__ sink,
+                        float *__restrict__ out, int packed) {
     __shared__ float red_m[MW][64];
     __shared__ float red_l[MW][64];
     __shared__ f32x4 red_a[MW][64];
@@ -698,9 +715,10 @@ mla_merge_frag16_kernel(const uint32_t *__restrict__ part_acc, const float *__re
             for (int r = 0; r < 4; r++) r4[r] += t[r];
         }
     }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
     const int head = hb * HB + n;
     if (head >= nh) return;
+    if (sink && mx > -INFINITY) l += __expf(sink[head] - mx);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; r++) r4[r] *= inv;
     // accumulator register i <-> dim 16 db + 4 g + i
@@ -708,13 +726,14 @@ mla_merge_frag16_kernel(const uint32_t *__restrict__ part_acc, const float *__re
 }
 
 int run(Params &p, hipStream_t s) {
-    static bool attr_set = false;
+    static std::once_flag attr_once;
+    static hipError_t attr_err = hipSuccess;
     const size_t smem = sizeof(Smem);
-    if (!attr_set) {
-        CWICK_HIP_CALL(hipFuncSetAttribute((const void *)mla_roles_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    std::call_once(attr_once, [&] {
+        attr_err = hipFuncSetAttribute((const void *)mla_roles_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    });
+    CWICK_HIP_CALL(attr_err);
     const int n_hb = (p.nh + HW - 1) / HW;
     const int64_t total = (int64_t)n_hb * p.n_splits * p.nq;
     CWICK_REQUIRE(total <= 0x7FFFFFFF, "mla: grid of %lld workgroups is too large", (long long)total);
@@ -735,22 +754,21 @@ int run(Params &p, hipStream_t s) {
         ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
         if (p.n_splits <= 8)
             mla_merge_frag16_kernel<<<dim3(2 * n_hb * 4, p.nq), 64 * 8, 0, s>>>(
-                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out, 1);
+                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 1);
         else
             mla_merge_frag16_kernel<<<dim3(2 * n_hb * NDB, p.nq), 64 * (p.n_splits <= 64 ? 8 : MW), 0, s>>>(
-                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.out, 0);
+                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 0);
         CWICK_HIP_CALL(hipGetLastError());
     }
     return 1;
 }
 
 int splits_per_cu() {
-    static int v = -1;
-    if (v < 0) {
+    static const int v = [] {
         const char *e = getenv("CWICK_HIP_MLA_WG_PER_CU");
-        v = e ? atoi(e) : 1;
-        if (v < 1 || v > 8) v = 1;
-    }
+        const int x = e ? atoi(e) : 1;
+        return (x < 1 || x > 8) ? 1 : x;
+    }();
     return v;
 }
 
@@ -758,8 +776,8 @@ int splits_per_cu() {
 
 int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
-                      int64_t n_list, const uint16_t *q, int n_heads, float scale, float *out,
-                      hipStream_t s) {
+                      int64_t n_list, const uint16_t *q, int n_heads, float scale, const float *sink,
+                      float *out, hipStream_t s) {
     CWICK_REQUIRE(rows && scales && q && out, "mla_decode: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 4096, "mla_decode: batch %d", batch);
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
@@ -776,7 +794,7 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
     Params p{};
     p.rows = rows; p.scales = scales; p.row_bstride = row_bstride; p.scale_bstride = scale_bstride;
     p.n_rows = n_rows; p.sel = sel; p.n_list = n_list; p.list_step = 0;
-    p.q = q; p.nh = n_heads; p.nq = batch; p.scale = scale; p.out = out;
+    p.q = q; p.nh = n_heads; p.nq = batch; p.scale = scale; p.out = out; p.sink = sink;
     // one workgroup is resident per CU: one round of workgroups
     const int n_hb = (n_heads + HW - 1) / HW;
     int64_t want = (int64_t)splits_per_cu() * num_cus() / ((int64_t)n_hb * batch);

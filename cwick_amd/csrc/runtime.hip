@@ -102,11 +102,9 @@ struct Scratch {
     void *p = nullptr;
     size_t cap = 0;
 };
-static std::unordered_map<hipStream_t, Scratch> g_ws, g_stage;
+static std::unordered_map<hipStream_t, Scratch> g_ws;
 
-static void *grow(std::unordered_map<hipStream_t, Scratch> &m, hipStream_t s, size_t bytes) {
-    std::lock_guard<std::mutex> lk(g_mu);
-    Scratch &b = m[s];
+static void *grow_one(Scratch &b, hipStream_t s, size_t bytes) {
     if (bytes <= b.cap) return b.p;
     // A buffer in use by kernels already enqueued on `s` must outlive them.
     if (b.p) {
@@ -124,8 +122,44 @@ static void *grow(std::unordered_map<hipStream_t, Scratch> &m, hipStream_t s, si
     return b.p;
 }
 
-void *workspace(hipStream_t s, size_t bytes) { return grow(g_ws, s, bytes); }
-void *staging(hipStream_t s, size_t bytes) { return grow(g_stage, s, bytes); }
+void *workspace(hipStream_t s, size_t bytes) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    return grow_one(g_ws[s], s, bytes);
+}
+
+// forget (and free) the workspace of a stream that is about to be destroyed
+static void drop_workspace(hipStream_t s) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_ws.find(s);
+    if (it == g_ws.end()) return;
+    if (it->second.p) (void)hipFree(it->second.p);
+    g_ws.erase(it);
+}
+
+// What a host-pointer call needs of its own: a stream and a staging buffer for the operands it
+// copies in and out.  Every cache handle owns one, so calls on different handles share nothing
+// (the split-K workspace is keyed by the stream) and may run on different threads; the calls
+// that take no handle share g_free_ctx under g_free_mu.
+struct HostCtx {
+    hipStream_t stream = nullptr;
+    Scratch stage;
+    bool init() {
+        return hip_ok(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking), "hipStreamCreate(handle)");
+    }
+    void *staging(size_t bytes) { return grow_one(stage, stream, bytes); }
+    void destroy() {
+        if (stream) {
+            (void)hipStreamSynchronize(stream);
+            drop_workspace(stream);
+            (void)hipStreamDestroy(stream);
+            stream = nullptr;
+        }
+        if (stage.p) (void)hipFree(stage.p);
+        stage = Scratch{};
+    }
+};
+static std::mutex g_free_mu;
+static HostCtx g_free_ctx;
 
 // ---------------------------------------------------------------------------
 // phase timers: event pairs around kernel launches, summed on read
@@ -185,9 +219,7 @@ static void prof_drain_locked() {
 static void free_all_scratch() {
     std::lock_guard<std::mutex> lk(g_mu);
     for (auto &kv : g_ws) if (kv.second.p) (void)hipFree(kv.second.p);
-    for (auto &kv : g_stage) if (kv.second.p) (void)hipFree(kv.second.p);
     g_ws.clear();
-    g_stage.clear();
 }
 
 }  // namespace cwick
@@ -201,28 +233,55 @@ struct cwick_hip_kv {
     int64_t capacity;
     int n_kv_heads, head_dim;
     uint16_t *k, *v;
+    HostCtx ctx;
 };
 struct cwick_hip_latent {
     int slots;
     int64_t capacity;
     uint8_t *rows;    // [slots][capacity][576]
     float *scales;    // [slots][capacity][5]
+    HostCtx ctx;
 };
 struct cwick_hip_ikeys {
     int slots;
     int64_t capacity;
     uint8_t *rows;    // [slots][capacity][128]
     float *scales;    // [slots][capacity]
+    HostCtx ctx;
 };
 
-// Stage `bytes` of host memory into the per-stream staging buffer at `off`.
-static void *stage_in(char *base, size_t &off, const void *host, size_t bytes) {
-    void *d = base + off;
-    off += (bytes + 255) & ~(size_t)255;
-    if (hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, nullptr) != hipSuccess) return nullptr;
-    return d;
-}
 static size_t pad256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// The operands of one host-pointer call, laid out in the context's staging buffer: in() copies
+// a host operand up on the context's stream, room() reserves space for a result, out() brings
+// a result back and waits for everything the call enqueued.
+struct Stager {
+    HostCtx &ctx;
+    char *base;
+    size_t off = 0;
+    bool ok;
+    Stager(HostCtx &c, size_t total) : ctx(c), base((char *)c.staging(total)), ok(base != nullptr) {}
+    template <class T>
+    T *in(const T *host, size_t bytes) {
+        if (!ok) return nullptr;
+        T *d = (T *)(base + off);
+        off += pad256(bytes);
+        if (!hip_ok(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, ctx.stream), "hipMemcpyAsync(operand)"))
+            ok = false;
+        return ok ? d : nullptr;
+    }
+    template <class T>
+    T *room(size_t bytes) {
+        if (!ok) return nullptr;
+        T *d = (T *)(base + off);
+        off += pad256(bytes);
+        return d;
+    }
+    bool out(void *host, const void *dev, size_t bytes) {
+        return hip_ok(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx.stream), "hipMemcpyAsync(result)");
+    }
+    bool wait() { return hip_ok(hipStreamSynchronize(ctx.stream), "hipStreamSynchronize(handle)"); }
+};
 
 extern "C" {
 
@@ -244,7 +303,16 @@ int cwick_hip_force(int on) {
 }
 
 void cwick_hip_shutdown(void) {
-    if (g_state == 1) (void)hipDeviceSynchronize();
+    bool up;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        up = g_state == 1;
+    }
+    if (up) (void)hipDeviceSynchronize();
+    {
+        std::lock_guard<std::mutex> lk(g_free_mu);
+        g_free_ctx.destroy();
+    }
     free_all_scratch();
 }
 
@@ -266,11 +334,12 @@ cwick_hip_kv *cwick_hip_kv_create(int64_t capacity, int n_kv_heads, int head_dim
                   (long long)capacity, n_kv_heads, head_dim);
         return nullptr;
     }
-    cwick_hip_kv *c = new cwick_hip_kv{capacity, n_kv_heads, head_dim, nullptr, nullptr};
+    cwick_hip_kv *c = new cwick_hip_kv{capacity, n_kv_heads, head_dim, nullptr, nullptr, {}};
     size_t bytes = (size_t)capacity * n_kv_heads * head_dim * sizeof(uint16_t);
-    if (!hip_ok(hipMalloc((void **)&c->k, bytes), "hipMalloc(K cache)") ||
+    if (!c->ctx.init() || !hip_ok(hipMalloc((void **)&c->k, bytes), "hipMalloc(K cache)") ||
         !hip_ok(hipMalloc((void **)&c->v, bytes), "hipMalloc(V cache)")) {
         if (c->k) (void)hipFree(c->k);
+        c->ctx.destroy();
         delete c;
         return nullptr;
     }
@@ -280,19 +349,24 @@ cwick_hip_kv *cwick_hip_kv_create(int64_t capacity, int n_kv_heads, int head_dim
 void cwick_hip_kv_free(cwick_hip_kv *c) {
     if (!c) return;
     (void)hipDeviceSynchronize();
+    c->ctx.destroy();
     (void)hipFree(c->k);
     (void)hipFree(c->v);
     delete c;
 }
 
+#define KV_RANGE_CHECK(what)                                                             \
+    if (!backend_ready()) return 0;   /* the reason is recorded */                                  \
+    CWICK_REQUIRE(c, what ": null handle");                                               \
+    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,                          \
+                  what ": rows %lld..%lld outside capacity %lld", (long long)pos0,       \
+                  (long long)(pos0 + n), (long long)c->capacity)
+
 int cwick_hip_kv_write(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *k_rows,
                        const uint16_t *v_rows) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
-    CWICK_REQUIRE(c && k_rows && v_rows, "kv_write: null argument");
-    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,
-                  "kv_write: rows %lld..%lld outside capacity %lld", (long long)pos0,
-                  (long long)(pos0 + n), (long long)c->capacity);
+    KV_RANGE_CHECK("kv_write");
+    CWICK_REQUIRE(k_rows && v_rows, "kv_write: null argument");
     size_t row = (size_t)c->n_kv_heads * c->head_dim;
     CWICK_HIP_CALL(hipMemcpy(c->k + pos0 * row, k_rows, n * row * 2, hipMemcpyHostToDevice));
     CWICK_HIP_CALL(hipMemcpy(c->v + pos0 * row, v_rows, n * row * 2, hipMemcpyHostToDevice));
@@ -302,22 +376,43 @@ int cwick_hip_kv_write(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t 
 int cwick_hip_kv_write_f32(cwick_hip_kv *c, int64_t pos0, int64_t n, const float *k_rows,
                            const float *v_rows) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
-    CWICK_REQUIRE(c && k_rows && v_rows, "kv_write_f32: null argument");
-    CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,
-                  "kv_write_f32: rows outside capacity");
+    KV_RANGE_CHECK("kv_write_f32");
+    CWICK_REQUIRE(k_rows && v_rows, "kv_write_f32: null argument");
     size_t row = (size_t)c->n_kv_heads * c->head_dim;
     size_t bytes = (size_t)n * row * sizeof(float);
-    char *st = (char *)staging(nullptr, 2 * pad256(bytes));
-    CWICK_REQUIRE(st, "kv_write_f32: staging allocation failed");
-    size_t off = 0;
-    float *dk = (float *)stage_in(st, off, k_rows, bytes);
-    float *dv = (float *)stage_in(st, off, v_rows, bytes);
+    Stager st(c->ctx, 2 * pad256(bytes));
+    CWICK_REQUIRE(st.ok, "kv_write_f32: staging allocation failed");
+    const float *dk = st.in(k_rows, bytes);
+    const float *dv = st.in(v_rows, bytes);
     CWICK_REQUIRE(dk && dv, "kv_write_f32: upload failed");
-    if (!launch_narrow_bf16(dk, n * row, c->k + pos0 * row, nullptr)) return 0;
-    if (!launch_narrow_bf16(dv, n * row, c->v + pos0 * row, nullptr)) return 0;
-    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
+    if (!launch_narrow_bf16(dk, n * row, c->k + pos0 * row, c->ctx.stream)) return 0;
+    if (!launch_narrow_bf16(dv, n * row, c->v + pos0 * row, c->ctx.stream)) return 0;
+    return st.wait() ? 1 : 0;
+}
+
+int cwick_hip_kv_read(cwick_hip_kv *c, int64_t pos0, int64_t n, uint16_t *k_rows, uint16_t *v_rows) {
+    clear_error();
+    KV_RANGE_CHECK("kv_read");
+    CWICK_REQUIRE(k_rows && v_rows, "kv_read: null argument");
+    size_t row = (size_t)c->n_kv_heads * c->head_dim;
+    CWICK_HIP_CALL(hipMemcpy(k_rows, c->k + pos0 * row, n * row * 2, hipMemcpyDeviceToHost));
+    CWICK_HIP_CALL(hipMemcpy(v_rows, c->v + pos0 * row, n * row * 2, hipMemcpyDeviceToHost));
     return 1;
+}
+
+int cwick_hip_kv_read_f32(cwick_hip_kv *c, int64_t pos0, int64_t n, float *k_rows, float *v_rows) {
+    clear_error();
+    KV_RANGE_CHECK("kv_read_f32");
+    CWICK_REQUIRE(k_rows && v_rows, "kv_read_f32: null argument");
+    size_t row = (size_t)c->n_kv_heads * c->head_dim;
+    size_t bytes = (size_t)n * row * sizeof(float);
+    Stager st(c->ctx, 2 * pad256(bytes));
+    CWICK_REQUIRE(st.ok, "kv_read_f32: staging allocation failed");
+    float *dk = st.room<float>(bytes), *dv = st.room<float>(bytes);
+    if (!launch_widen_bf16(c->k + pos0 * row, n * row, dk, c->ctx.stream)) return 0;
+    if (!launch_widen_bf16(c->v + pos0 * row, n * row, dv, c->ctx.stream)) return 0;
+    if (!st.out(k_rows, dk, bytes) || !st.out(v_rows, dv, bytes)) return 0;
+    return st.wait() ? 1 : 0;
 }
 
 uint16_t *cwick_hip_kv_k_dev(cwick_hip_kv *c) { return c ? c->k : nullptr; }
@@ -331,13 +426,15 @@ cwick_hip_latent *cwick_hip_latent_create(int slots, int64_t capacity) {
         set_error("latent_create: slots %d capacity %lld", slots, (long long)capacity);
         return nullptr;
     }
-    cwick_hip_latent *c = new cwick_hip_latent{slots, capacity, nullptr, nullptr};
+    cwick_hip_latent *c = new cwick_hip_latent{slots, capacity, nullptr, nullptr, {}};
     size_t rows = (size_t)slots * capacity;
     // 64 bytes of slack: the kernels read rows in 16-byte pieces
-    if (!hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_LATENT_KDIM + 64), "hipMalloc(latent)") ||
+    if (!c->ctx.init() ||
+        !hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_LATENT_KDIM + 64), "hipMalloc(latent)") ||
         !hip_ok(hipMalloc((void **)&c->scales, rows * CWICK_HIP_LATENT_NBLK * sizeof(float) + 64),
                 "hipMalloc(latent scales)")) {
         if (c->rows) (void)hipFree(c->rows);
+        c->ctx.destroy();
         delete c;
         return nullptr;
     }
@@ -347,13 +444,14 @@ cwick_hip_latent *cwick_hip_latent_create(int slots, int64_t capacity) {
 void cwick_hip_latent_free(cwick_hip_latent *c) {
     if (!c) return;
     (void)hipDeviceSynchronize();
+    c->ctx.destroy();
     (void)hipFree(c->rows);
     (void)hipFree(c->scales);
     delete c;
 }
 
 #define LATENT_RANGE_CHECK(what)                                                          \
-    CWICK_REQUIRE(backend_ready(), "backend not ready");                                  \
+    if (!backend_ready()) return 0;   /* the reason is recorded */                                  \
     CWICK_REQUIRE(c, what ": null handle");                                               \
     CWICK_REQUIRE(slot >= 0 && slot < c->slots, what ": slot %d of %d", slot, c->slots);  \
     CWICK_REQUIRE(pos0 >= 0 && n > 0 && pos0 + n <= c->capacity,                          \
@@ -380,17 +478,15 @@ int cwick_hip_latent_write_f32(cwick_hip_latent *c, int slot, int64_t pos0, int6
     LATENT_RANGE_CHECK("latent_write_f32");
     CWICK_REQUIRE(rows, "latent_write_f32: null argument");
     size_t bytes = (size_t)n * CWICK_HIP_LATENT_KDIM * sizeof(float);
-    char *st = (char *)staging(nullptr, pad256(bytes));
-    CWICK_REQUIRE(st, "latent_write_f32: staging allocation failed");
-    size_t off = 0;
-    float *d = (float *)stage_in(st, off, rows, bytes);
+    Stager st(c->ctx, pad256(bytes));
+    CWICK_REQUIRE(st.ok, "latent_write_f32: staging allocation failed");
+    const float *d = st.in(rows, bytes);
     CWICK_REQUIRE(d, "latent_write_f32: upload failed");
     size_t r0 = (size_t)slot * c->capacity + pos0;
     if (!launch_quant_latent(d, n, c->rows + r0 * CWICK_HIP_LATENT_KDIM,
-                             c->scales + r0 * CWICK_HIP_LATENT_NBLK, nullptr))
+                             c->scales + r0 * CWICK_HIP_LATENT_NBLK, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
-    return 1;
+    return st.wait() ? 1 : 0;
 }
 
 int cwick_hip_latent_read(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n, uint8_t *rows,
@@ -424,11 +520,13 @@ cwick_hip_ikeys *cwick_hip_ikeys_create(int slots, int64_t capacity) {
         set_error("ikeys_create: slots %d capacity %lld", slots, (long long)capacity);
         return nullptr;
     }
-    cwick_hip_ikeys *c = new cwick_hip_ikeys{slots, capacity, nullptr, nullptr};
+    cwick_hip_ikeys *c = new cwick_hip_ikeys{slots, capacity, nullptr, nullptr, {}};
     size_t rows = (size_t)slots * capacity;
-    if (!hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_INDEX_DIM + 64), "hipMalloc(ikeys)") ||
+    if (!c->ctx.init() ||
+        !hip_ok(hipMalloc((void **)&c->rows, rows * CWICK_HIP_INDEX_DIM + 64), "hipMalloc(ikeys)") ||
         !hip_ok(hipMalloc((void **)&c->scales, rows * sizeof(float) + 64), "hipMalloc(ikey scales)")) {
         if (c->rows) (void)hipFree(c->rows);
+        c->ctx.destroy();
         delete c;
         return nullptr;
     }
@@ -438,6 +536,7 @@ cwick_hip_ikeys *cwick_hip_ikeys_create(int slots, int64_t capacity) {
 void cwick_hip_ikeys_free(cwick_hip_ikeys *c) {
     if (!c) return;
     (void)hipDeviceSynchronize();
+    c->ctx.destroy();
     (void)hipFree(c->rows);
     (void)hipFree(c->scales);
     delete c;
@@ -462,15 +561,25 @@ int cwick_hip_ikeys_write_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_
     LATENT_RANGE_CHECK("ikeys_write_f32");
     CWICK_REQUIRE(rows, "ikeys_write_f32: null argument");
     size_t bytes = (size_t)n * CWICK_HIP_INDEX_DIM * sizeof(float);
-    char *st = (char *)staging(nullptr, pad256(bytes));
-    CWICK_REQUIRE(st, "ikeys_write_f32: staging allocation failed");
-    size_t off = 0;
-    float *d = (float *)stage_in(st, off, rows, bytes);
+    Stager st(c->ctx, pad256(bytes));
+    CWICK_REQUIRE(st.ok, "ikeys_write_f32: staging allocation failed");
+    const float *d = st.in(rows, bytes);
     CWICK_REQUIRE(d, "ikeys_write_f32: upload failed");
     size_t r0 = (size_t)slot * c->capacity + pos0;
-    if (!launch_quant_ikeys(d, n, c->rows + r0 * CWICK_HIP_INDEX_DIM, c->scales + r0, nullptr))
+    if (!launch_quant_ikeys(d, n, c->rows + r0 * CWICK_HIP_INDEX_DIM, c->scales + r0, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipStreamSynchronize(nullptr));
+    return st.wait() ? 1 : 0;
+}
+
+int cwick_hip_ikeys_read(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n, uint8_t *rows,
+                         float *scales) {
+    clear_error();
+    LATENT_RANGE_CHECK("ikeys_read");
+    CWICK_REQUIRE(rows && scales, "ikeys_read: null argument");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    CWICK_HIP_CALL(hipMemcpy(rows, c->rows + r0 * CWICK_HIP_INDEX_DIM, (size_t)n * CWICK_HIP_INDEX_DIM,
+                             hipMemcpyDeviceToHost));
+    CWICK_HIP_CALL(hipMemcpy(scales, c->scales + r0, (size_t)n * sizeof(float), hipMemcpyDeviceToHost));
     return 1;
 }
 
@@ -488,7 +597,7 @@ int cwick_hip_gqa_decode_dev(const uint16_t *k, const uint16_t *v, int64_t n_key
                              int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
                              void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_gqa_decode(k, v, n_keys, n_kv_heads, head_dim, q, n_heads, scale, out,
                              (hipStream_t)stream);
 }
@@ -497,7 +606,7 @@ int cwick_hip_gqa_prefill_dev(const uint16_t *k, const uint16_t *v, int64_t pos0
                               int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
                               float scale, float *out, void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_gqa_prefill(k, v, pos0, n, n_kv_heads, head_dim, q, n_heads, scale, out,
                               (hipStream_t)stream);
 }
@@ -507,16 +616,26 @@ int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales, int64_t r
                              int64_t n_list, const uint16_t *q, int n_heads, float scale,
                              float *out, void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_rows, batch, sel,
-                             n_list, q, n_heads, scale, out, (hipStream_t)stream);
+                             n_list, q, n_heads, scale, nullptr, out, (hipStream_t)stream);
+}
+
+int cwick_hip_mla_decode_sink_dev(const uint8_t *rows, const float *scales, int64_t row_batch_stride,
+                                  int64_t scale_batch_stride, int64_t n_rows, int batch,
+                                  const int32_t *sel, int64_t n_list, const uint16_t *q, int n_heads,
+                                  float scale, const float *sink, float *out, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_rows, batch, sel,
+                             n_list, q, n_heads, scale, sink, out, (hipStream_t)stream);
 }
 
 int cwick_hip_mla_prefill_chunk_dev(const uint8_t *rows, const float *scales, int64_t pos0,
                                     int64_t n, const uint16_t *q, int n_heads, float scale,
                                     float *out, void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_mla_prefill(rows, scales, pos0, n, q, n_heads, scale, out, (hipStream_t)stream);
 }
 
@@ -525,15 +644,25 @@ int cwick_hip_indexer_scores_dev(const uint8_t *keys, const float *kscale, int64
                                  const uint16_t *q_idx, const float *w, int n_idx_heads,
                                  float *scores, void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_indexer_scores(keys, kscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
-                                 q_idx, w, n_idx_heads, scores, (hipStream_t)stream);
+                                 q_idx, w, n_idx_heads, CWICK_HIP_INDEXER_GLM, scores, (hipStream_t)stream);
+}
+
+int cwick_hip_indexer_scores_mode_dev(const uint8_t *keys, const float *kscale, int64_t key_batch_stride,
+                                      int64_t kscale_batch_stride, int batch, int64_t n_keys,
+                                      const uint16_t *q_idx, const float *w, int n_idx_heads, int mode,
+                                      float *scores, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_indexer_scores(keys, kscale, key_batch_stride, kscale_batch_stride, batch, n_keys,
+                                 q_idx, w, n_idx_heads, mode, scores, (hipStream_t)stream);
 }
 
 int cwick_hip_topk_dev(const float *scores, int batch, int64_t n, int64_t k, int32_t *out_idx,
                        void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_topk(scores, batch, n, k, out_idx, (hipStream_t)stream);
 }
 
@@ -544,7 +673,7 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale, int64_t
                              int64_t topk, const uint16_t *q, int n_heads, float scale,
                              float *scores_tmp, int32_t *sel_out, float *out, void *stream) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(scores_tmp && sel_out, "dsa_decode_dev: scores_tmp and sel_out are required");
     CWICK_REQUIRE(topk > 0 && n_keys > 0, "dsa_decode_dev: topk %lld n_keys %lld",
                   (long long)topk, (long long)n_keys);
@@ -562,59 +691,55 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale, int64_t
             return 0;
     } else {
         if (!launch_indexer_scores(ikeys, ikscale, key_batch_stride, kscale_batch_stride, batch,
-                                   n_keys, q_idx, w, n_idx_heads, scores_tmp, s))
+                                   n_keys, q_idx, w, n_idx_heads, CWICK_HIP_INDEXER_GLM, scores_tmp, s))
             return 0;
         if (!launch_topk(scores_tmp, batch, n_keys, topk, sel_out, s)) return 0;
     }
     // rows past min(topk, n_keys) are -1 and are skipped by the attention kernel
     return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_keys, batch,
-                             sel_out, topk, q, n_heads, scale, out, s);
+                             sel_out, topk, q, n_heads, scale, nullptr, out, s);
 }
 
 // ---- host-pointer entry points -------------------------------------------------
 int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q, int n_heads,
                          float scale, float *out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q && out, "gqa_decode: null argument");
     CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "gqa_decode: n_keys %lld, capacity %lld",
                   (long long)n_keys, (long long)c->capacity);
     CWICK_REQUIRE(n_heads > 0 && n_heads <= 1024, "gqa_decode: n_heads %d", n_heads);
     size_t qb = (size_t)n_heads * c->head_dim * 2, ob = (size_t)n_heads * c->head_dim * 4;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
-    CWICK_REQUIRE(st, "gqa_decode: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    Stager st(c->ctx, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "gqa_decode: staging allocation failed");
+    const uint16_t *dq = st.in(q, qb);
     CWICK_REQUIRE(dq, "gqa_decode: upload failed");
-    float *dout = (float *)(st + off);
+    float *dout = st.room<float>(ob);
     if (!launch_gqa_decode(c->k, c->v, n_keys, c->n_kv_heads, c->head_dim, dq, n_heads, scale, dout,
-                           nullptr))
+                           c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
-    return 1;
+    return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
 int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *q, int n_heads,
                           float scale, float *out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q && out, "gqa_prefill: null argument");
     CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= c->capacity,
                   "gqa_prefill: positions %lld..%lld outside capacity %lld", (long long)pos0,
                   (long long)(pos0 + n), (long long)c->capacity);
     CWICK_REQUIRE(n_heads > 0 && n_heads <= 1024, "gqa_prefill: n_heads %d", n_heads);
     size_t qb = (size_t)n * n_heads * c->head_dim * 2, ob = (size_t)n * n_heads * c->head_dim * 4;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
-    CWICK_REQUIRE(st, "gqa_prefill: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    Stager st(c->ctx, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "gqa_prefill: staging allocation failed");
+    const uint16_t *dq = st.in(q, qb);
     CWICK_REQUIRE(dq, "gqa_prefill: upload failed");
-    float *dout = (float *)(st + off);
+    float *dout = st.room<float>(ob);
     if (!launch_gqa_prefill(c->k, c->v, pos0, n, c->n_kv_heads, c->head_dim, dq, n_heads, scale,
-                            dout, nullptr))
+                            dout, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
-    return 1;
+    return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
 // sel entries must address rows of the slot; checked on the host because a bad
@@ -631,8 +756,14 @@ static int check_sel(const int32_t *sel, int64_t n, int64_t capacity) {
 
 int cwick_hip_mla_decode(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
                          const uint16_t *q, int n_heads, float scale, float *out) {
+    return cwick_hip_mla_decode_sink(c, slot, sel, n_list, q, n_heads, scale, nullptr, out);
+}
+
+int cwick_hip_mla_decode_sink(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
+                              const uint16_t *q, int n_heads, float scale, const float *sink,
+                              float *out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q && out, "mla_decode: null argument");
     CWICK_REQUIRE(slot >= 0 && slot < c->slots, "mla_decode: slot %d of %d", slot, c->slots);
     CWICK_REQUIRE(n_list >= 1, "mla_decode: n_list %lld", (long long)n_list);
@@ -643,24 +774,25 @@ int cwick_hip_mla_decode(cwick_hip_latent *c, int slot, const int32_t *sel, int6
     size_t qb = (size_t)n_heads * CWICK_HIP_LATENT_KDIM * 2;
     size_t ob = (size_t)n_heads * CWICK_HIP_LATENT_VDIM * 4;
     size_t sb = sel ? (size_t)n_list * 4 : 0;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob) + pad256(sb));
-    CWICK_REQUIRE(st, "mla_decode: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
-    int32_t *dsel = sel ? (int32_t *)stage_in(st, off, sel, sb) : nullptr;
-    CWICK_REQUIRE(dq && (!sel || dsel), "mla_decode: upload failed");
-    float *dout = (float *)(st + off);
+    size_t kb = sink ? (size_t)n_heads * 4 : 0;
+    Stager st(c->ctx, pad256(qb) + pad256(ob) + pad256(sb) + pad256(kb));
+    CWICK_REQUIRE(st.ok, "mla_decode: staging allocation failed");
+    const uint16_t *dq = st.in(q, qb);
+    const int32_t *dsel = sel ? st.in(sel, sb) : nullptr;
+    const float *dsink = sink ? st.in(sink, kb) : nullptr;
+    CWICK_REQUIRE(dq && (!sel || dsel) && (!sink || dsink), "mla_decode: upload failed");
+    float *dout = st.room<float>(ob);
     if (!launch_mla_decode(cwick_hip_latent_rows_dev(c, slot), cwick_hip_latent_scales_dev(c, slot),
-                           0, 0, c->capacity, 1, dsel, n_list, dq, n_heads, scale, dout, nullptr))
+                           0, 0, c->capacity, 1, dsel, n_list, dq, n_heads, scale, dsink, dout,
+                           c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
-    return 1;
+    return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
 int cwick_hip_mla_prefill_chunk(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
                                 const uint16_t *q, int n_heads, float scale, float *out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q && out, "mla_prefill_chunk: null argument");
     CWICK_REQUIRE(slot >= 0 && slot < c->slots, "mla_prefill_chunk: slot %d of %d", slot, c->slots);
     CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= c->capacity,
@@ -669,23 +801,27 @@ int cwick_hip_mla_prefill_chunk(cwick_hip_latent *c, int slot, int64_t pos0, int
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_prefill_chunk: n_heads %d (1..128)", n_heads);
     size_t qb = (size_t)n * n_heads * CWICK_HIP_LATENT_KDIM * 2;
     size_t ob = (size_t)n * n_heads * CWICK_HIP_LATENT_VDIM * 4;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(ob));
-    CWICK_REQUIRE(st, "mla_prefill_chunk: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    Stager st(c->ctx, pad256(qb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "mla_prefill_chunk: staging allocation failed");
+    const uint16_t *dq = st.in(q, qb);
     CWICK_REQUIRE(dq, "mla_prefill_chunk: upload failed");
-    float *dout = (float *)(st + off);
+    float *dout = st.room<float>(ob);
     if (!launch_mla_prefill(cwick_hip_latent_rows_dev(c, slot), cwick_hip_latent_scales_dev(c, slot),
-                            pos0, n, dq, n_heads, scale, dout, nullptr))
+                            pos0, n, dq, n_heads, scale, dout, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
-    return 1;
+    return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
 int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys, const uint16_t *q_idx,
                              const float *w, int n_idx_heads, float *scores) {
+    return cwick_hip_indexer_scores_mode(c, slot, n_keys, q_idx, w, n_idx_heads, CWICK_HIP_INDEXER_GLM,
+                                         scores);
+}
+
+int cwick_hip_indexer_scores_mode(cwick_hip_ikeys *c, int slot, int64_t n_keys, const uint16_t *q_idx,
+                                  const float *w, int n_idx_heads, int mode, float *scores) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q_idx && w && scores, "indexer_scores: null argument");
     CWICK_REQUIRE(slot >= 0 && slot < c->slots, "indexer_scores: slot %d of %d", slot, c->slots);
     CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "indexer_scores: n_keys %lld, capacity %lld",
@@ -694,25 +830,23 @@ int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys, const
                   n_idx_heads);
     size_t qb = (size_t)n_idx_heads * CWICK_HIP_INDEX_DIM * 2, wb = (size_t)n_idx_heads * 4;
     size_t ob = (size_t)n_keys * 4;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(wb) + pad256(ob));
-    CWICK_REQUIRE(st, "indexer_scores: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q_idx, qb);
-    float *dw = (float *)stage_in(st, off, w, wb);
+    Stager st(c->ctx, pad256(qb) + pad256(wb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "indexer_scores: staging allocation failed");
+    const uint16_t *dq = st.in(q_idx, qb);
+    const float *dw = st.in(w, wb);
     CWICK_REQUIRE(dq && dw, "indexer_scores: upload failed");
-    float *dout = (float *)(st + off);
+    float *dout = st.room<float>(ob);
     if (!launch_indexer_scores(cwick_hip_ikeys_rows_dev(c, slot), cwick_hip_ikeys_scales_dev(c, slot),
-                               0, 0, 1, n_keys, dq, dw, n_idx_heads, dout, nullptr))
+                               0, 0, 1, n_keys, dq, dw, n_idx_heads, mode, dout, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(scores, dout, ob, hipMemcpyDeviceToHost));
-    return 1;
+    return st.out(scores, dout, ob) && st.wait() ? 1 : 0;
 }
 
 int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys,
                                     const uint16_t *q_idx, const float *w, int n_idx_heads,
                                     float *scores, float *bound) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(c && q_idx && w && scores && bound, "indexer_scores_approx: null argument");
     CWICK_REQUIRE(slot >= 0 && slot < c->slots, "indexer_scores_approx: slot %d of %d", slot, c->slots);
     CWICK_REQUIRE(n_keys >= 1 && n_keys <= c->capacity, "indexer_scores_approx: n_keys %lld, capacity %lld",
@@ -722,21 +856,19 @@ int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys
     const int n_slots = indexer_approx_slots(n_keys);
     size_t qb = (size_t)n_idx_heads * CWICK_HIP_INDEX_DIM * 2, wb = (size_t)n_idx_heads * 4;
     size_t ob = (size_t)n_keys * 4, bb = (size_t)n_slots * 4;
-    char *st = (char *)staging(nullptr, pad256(qb) + pad256(wb) + pad256(ob) + pad256(bb) + 256);
-    CWICK_REQUIRE(st, "indexer_scores_approx: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q_idx, qb);
-    float *dw = (float *)stage_in(st, off, w, wb);
+    Stager st(c->ctx, pad256(qb) + pad256(wb) + pad256(ob) + pad256(bb) + 256);
+    CWICK_REQUIRE(st.ok, "indexer_scores_approx: staging allocation failed");
+    const uint16_t *dq = st.in(q_idx, qb);
+    const float *dw = st.in(w, wb);
     CWICK_REQUIRE(dq && dw, "indexer_scores_approx: upload failed");
-    float *dout = (float *)(st + off);
-    float *dbeta = (float *)(st + off + pad256(ob));
-    IndexerBandRow *drow = (IndexerBandRow *)(st + off + pad256(ob) + pad256(bb));
+    float *dout = st.room<float>(ob);
+    float *dbeta = st.room<float>(bb);
+    IndexerBandRow *drow = st.room<IndexerBandRow>(256);
     if (!launch_indexer_approx(cwick_hip_ikeys_rows_dev(c, slot), cwick_hip_ikeys_scales_dev(c, slot), 0, 0,
-                               1, n_keys, dq, dw, n_idx_heads, dout, dbeta, drow, nullptr, 0, nullptr))
+                               1, n_keys, dq, dw, n_idx_heads, dout, dbeta, drow, nullptr, 0, c->ctx.stream))
         return 0;
-    CWICK_HIP_CALL(hipMemcpy(scores, dout, ob, hipMemcpyDeviceToHost));
     std::vector<float> hb((size_t)n_slots);
-    CWICK_HIP_CALL(hipMemcpy(hb.data(), dbeta, bb, hipMemcpyDeviceToHost));
+    if (!st.out(scores, dout, ob) || !st.out(hb.data(), dbeta, bb) || !st.wait()) return 0;
     float m = hb[0];
     for (int i = 1; i < n_slots; i++) m = (hb[i] <= m) ? m : hb[i];      // NaN sticks
     *bound = m;
@@ -745,20 +877,22 @@ int cwick_hip_indexer_scores_approx(cwick_hip_ikeys *c, int slot, int64_t n_keys
 
 int cwick_hip_topk(const float *scores, int64_t n, int64_t k, int32_t *out_idx, int64_t *n_out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(scores && out_idx, "topk: null argument");
     CWICK_REQUIRE(n >= 1 && n <= ((int64_t)1 << 24), "topk: n %lld (1..2^24)", (long long)n);
     CWICK_REQUIRE(k >= 1 && k <= 65536, "topk: k %lld (1..65536)", (long long)k);
+    // no handle: the calls without one share a context and take turns
+    std::lock_guard<std::mutex> lk(g_free_mu);
+    if (!g_free_ctx.stream) CWICK_REQUIRE(g_free_ctx.init(), "topk: no stream");
     size_t sb = (size_t)n * 4, ob = (size_t)k * 4;
-    char *st = (char *)staging(nullptr, pad256(sb) + pad256(ob));
-    CWICK_REQUIRE(st, "topk: staging allocation failed");
-    size_t off = 0;
-    float *ds = (float *)stage_in(st, off, scores, sb);
+    Stager st(g_free_ctx, pad256(sb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "topk: staging allocation failed");
+    const float *ds = st.in(scores, sb);
     CWICK_REQUIRE(ds, "topk: upload failed");
-    int32_t *dout = (int32_t *)(st + off);
-    if (!launch_topk(ds, 1, n, k, dout, nullptr)) return 0;
+    int32_t *dout = st.room<int32_t>(ob);
+    if (!launch_topk(ds, 1, n, k, dout, g_free_ctx.stream)) return 0;
     int64_t got = k < n ? k : n;
-    CWICK_HIP_CALL(hipMemcpy(out_idx, dout, (size_t)got * 4, hipMemcpyDeviceToHost));
+    if (!st.out(out_idx, dout, (size_t)got * 4) || !st.wait()) return 0;
     if (n_out) *n_out = got;
     return 1;
 }
@@ -768,7 +902,7 @@ int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, 
                          int n_idx_heads, int64_t topk, const uint16_t *q, int n_heads, float scale,
                          float *out, int32_t *sel_out) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(ik && lat && q_idx && w && q && out, "dsa_decode: null argument");
     CWICK_REQUIRE(batch >= 1 && batch <= 1024, "dsa_decode: batch %d", batch);
     CWICK_REQUIRE(slot_step == 0 || slot_step == 1, "dsa_decode: slot_step %d (0 or 1)", slot_step);
@@ -785,28 +919,27 @@ int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, 
     size_t qb = (size_t)batch * n_heads * CWICK_HIP_LATENT_KDIM * 2;
     size_t scb = (size_t)batch * n_keys * 4, selb = (size_t)batch * topk * 4;
     size_t ob = (size_t)batch * n_heads * CWICK_HIP_LATENT_VDIM * 4;
-    char *st = (char *)staging(nullptr, pad256(qib) + pad256(wb) + pad256(qb) + pad256(scb) +
-                                            pad256(selb) + pad256(ob));
-    CWICK_REQUIRE(st, "dsa_decode: staging allocation failed");
-    size_t off = 0;
-    uint16_t *dqi = (uint16_t *)stage_in(st, off, q_idx, qib);
-    float *dw = (float *)stage_in(st, off, w, wb);
-    uint16_t *dq = (uint16_t *)stage_in(st, off, q, qb);
+    // the call runs on the latent cache's context (stream, staging)
+    Stager st(lat->ctx, pad256(qib) + pad256(wb) + pad256(qb) + pad256(scb) + pad256(selb) + pad256(ob));
+    CWICK_REQUIRE(st.ok, "dsa_decode: staging allocation failed");
+    const uint16_t *dqi = st.in(q_idx, qib);
+    const float *dw = st.in(w, wb);
+    const uint16_t *dq = st.in(q, qb);
     CWICK_REQUIRE(dqi && dw && dq, "dsa_decode: upload failed");
-    float *dsc = (float *)(st + off); off += pad256(scb);
-    int32_t *dsel = (int32_t *)(st + off); off += pad256(selb);
-    float *dout = (float *)(st + off);
+    float *dsc = st.room<float>(scb);
+    int32_t *dsel = st.room<int32_t>(selb);
+    float *dout = st.room<float>(ob);
     int ok = cwick_hip_dsa_decode_dev(
         cwick_hip_ikeys_rows_dev(ik, slot0), cwick_hip_ikeys_scales_dev(ik, slot0),
         (int64_t)slot_step * ik->capacity * CWICK_HIP_INDEX_DIM, (int64_t)slot_step * ik->capacity,
         cwick_hip_latent_rows_dev(lat, slot0), cwick_hip_latent_scales_dev(lat, slot0),
         (int64_t)slot_step * lat->capacity * CWICK_HIP_LATENT_KDIM,
         (int64_t)slot_step * lat->capacity * CWICK_HIP_LATENT_NBLK, batch, n_keys, dqi, dw,
-        n_idx_heads, topk, dq, n_heads, scale, dsc, dsel, dout, nullptr);
+        n_idx_heads, topk, dq, n_heads, scale, dsc, dsel, dout, lat->ctx.stream);
     if (!ok) return 0;
-    CWICK_HIP_CALL(hipMemcpy(out, dout, ob, hipMemcpyDeviceToHost));
-    if (sel_out) CWICK_HIP_CALL(hipMemcpy(sel_out, dsel, selb, hipMemcpyDeviceToHost));
-    return 1;
+    if (!st.out(out, dout, ob)) return 0;
+    if (sel_out && !st.out(sel_out, dsel, selb)) return 0;
+    return st.wait() ? 1 : 0;
 }
 
 void cwick_hip_prof_enable(int on) {
@@ -842,13 +975,15 @@ const char *cwick_hip_prof_name(int which) {
 
 int cwick_hip_e4m3_table(float *out256) {
     clear_error();
-    CWICK_REQUIRE(backend_ready(), "backend not ready");
+    if (!backend_ready()) return 0;   /* the reason is recorded */
     CWICK_REQUIRE(out256, "e4m3_table: null argument");
-    float *d = (float *)staging(nullptr, 1024);
-    CWICK_REQUIRE(d, "e4m3_table: staging allocation failed");
-    if (!launch_e4m3_table(d, nullptr)) return 0;
-    CWICK_HIP_CALL(hipMemcpy(out256, d, 1024, hipMemcpyDeviceToHost));
-    return 1;
+    std::lock_guard<std::mutex> lk(g_free_mu);
+    if (!g_free_ctx.stream) CWICK_REQUIRE(g_free_ctx.init(), "e4m3_table: no stream");
+    Stager st(g_free_ctx, 1024);
+    CWICK_REQUIRE(st.ok, "e4m3_table: staging allocation failed");
+    float *d = st.room<float>(1024);
+    if (!launch_e4m3_table(d, g_free_ctx.stream)) return 0;
+    return st.out(out256, d, 1024) && st.wait() ? 1 : 0;
 }
 
 }  // extern "C"

@@ -38,6 +38,8 @@ SIGNATURES = {
     "cwick_hip_kv_free": (None, [_vp]),
     "cwick_hip_kv_write": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "cwick_hip_kv_write_f32": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "cwick_hip_kv_read": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "cwick_hip_kv_read_f32": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "cwick_hip_kv_k_dev": (_vp, [_vp]),
     "cwick_hip_kv_v_dev": (_vp, [_vp]),
     "cwick_hip_latent_create": (_vp, [_int, _i64]),
@@ -51,13 +53,16 @@ SIGNATURES = {
     "cwick_hip_ikeys_free": (None, [_vp]),
     "cwick_hip_ikeys_write": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "cwick_hip_ikeys_write_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
+    "cwick_hip_ikeys_read": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "cwick_hip_ikeys_rows_dev": (_vp, [_vp, _int]),
     "cwick_hip_ikeys_scales_dev": (_vp, [_vp, _int]),
     "cwick_hip_gqa_decode": (_int, [_vp, _i64, _vp, _int, _flt, _vp]),
     "cwick_hip_gqa_prefill": (_int, [_vp, _i64, _i64, _vp, _int, _flt, _vp]),
     "cwick_hip_mla_decode": (_int, [_vp, _int, _vp, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_mla_decode_sink": (_int, [_vp, _int, _vp, _i64, _vp, _int, _flt, _vp, _vp]),
     "cwick_hip_mla_prefill_chunk": (_int, [_vp, _int, _i64, _i64, _vp, _int, _flt, _vp]),
     "cwick_hip_indexer_scores": (_int, [_vp, _int, _i64, _vp, _vp, _int, _vp]),
+    "cwick_hip_indexer_scores_mode": (_int, [_vp, _int, _i64, _vp, _vp, _int, _int, _vp]),
     "cwick_hip_indexer_scores_approx": (_int, [_vp, _int, _i64, _vp, _vp, _int, _vp, C.POINTER(_flt)]),
     "cwick_hip_topk": (_int, [_vp, _i64, _i64, _vp, C.POINTER(_i64)]),
     "cwick_hip_dsa_decode": (_int, [_vp, _vp, _int, _int, _int, _i64, _vp, _vp, _int, _i64,
@@ -67,9 +72,13 @@ SIGNATURES = {
                                          _vp, _vp]),
     "cwick_hip_mla_decode_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
                                         _flt, _vp, _vp]),
+    "cwick_hip_mla_decode_sink_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
+                                             _flt, _vp, _vp, _vp]),
     "cwick_hip_mla_prefill_chunk_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _flt, _vp, _vp]),
     "cwick_hip_indexer_scores_dev": (_int, [_vp, _vp, _i64, _i64, _int, _i64, _vp, _vp, _int,
                                             _vp, _vp]),
+    "cwick_hip_indexer_scores_mode_dev": (_int, [_vp, _vp, _i64, _i64, _int, _i64, _vp, _vp, _int,
+                                                 _int, _vp, _vp]),
     "cwick_hip_topk_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "cwick_hip_dsa_decode_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _int, _i64,
                                         _vp, _vp, _int, _i64, _vp, _int, _flt, _vp, _vp, _vp,
@@ -165,6 +174,20 @@ class KVCache:
         v, vp = _np(v_rows, np.float32)
         _check(lib().cwick_hip_kv_write_f32(self.h, pos0, k.shape[0], kp, vp), "kv_write_f32")
 
+    def read(self, pos0, n):
+        row = self.n_kv_heads * self.head_dim
+        k = np.empty((n, row), np.uint16)
+        v = np.empty((n, row), np.uint16)
+        _check(lib().cwick_hip_kv_read(self.h, pos0, n, k.ctypes.data, v.ctypes.data), "kv_read")
+        return k, v
+
+    def read_f32(self, pos0, n):
+        row = self.n_kv_heads * self.head_dim
+        k = np.empty((n, row), np.float32)
+        v = np.empty((n, row), np.float32)
+        _check(lib().cwick_hip_kv_read_f32(self.h, pos0, n, k.ctypes.data, v.ctypes.data), "kv_read_f32")
+        return k, v
+
     def k_dev(self):
         return lib().cwick_hip_kv_k_dev(self.h)
 
@@ -241,6 +264,13 @@ class IndexKeys:
         _check(lib().cwick_hip_ikeys_write_f32(self.h, slot, pos0, r.shape[0], rp),
                "ikeys_write_f32")
 
+    def read(self, slot, pos0, n):
+        rows = np.empty((n, IDIM), np.uint8)
+        scales = np.empty(n, np.float32)
+        _check(lib().cwick_hip_ikeys_read(self.h, slot, pos0, n, rows.ctypes.data,
+                                          scales.ctypes.data), "ikeys_read")
+        return rows, scales
+
     def rows_dev(self, slot=0):
         return lib().cwick_hip_ikeys_rows_dev(self.h, slot)
 
@@ -278,7 +308,7 @@ def gqa_prefill(cache, pos0, q, scale, raw=False):
     return out
 
 
-def mla_decode(cache, slot, q, scale, sel=None, n_list=None, raw=False):
+def mla_decode(cache, slot, q, scale, sel=None, n_list=None, raw=False, sink=None):
     q, qp = _np(q, np.uint16)
     nh = q.shape[0]
     assert q.shape[1] == KDIM
@@ -287,7 +317,13 @@ def mla_decode(cache, slot, q, scale, sel=None, n_list=None, raw=False):
         sel, selp = _np(sel, np.int32)
         n_list = sel.size if n_list is None else n_list
     out = np.empty((nh, VDIM), np.float32)
-    rc = lib().cwick_hip_mla_decode(cache.h, slot, selp, n_list, qp, nh, scale, out.ctypes.data)
+    if sink is not None:
+        sink, sinkp = _np(sink, np.float32)
+        assert sink.size == nh
+        rc = lib().cwick_hip_mla_decode_sink(cache.h, slot, selp, n_list, qp, nh, scale, sinkp,
+                                             out.ctypes.data)
+    else:
+        rc = lib().cwick_hip_mla_decode(cache.h, slot, selp, n_list, qp, nh, scale, out.ctypes.data)
     if raw:
         return rc, out
     _check(rc, "mla_decode")
@@ -306,12 +342,19 @@ def mla_prefill_chunk(cache, slot, pos0, q, scale, raw=False):
     return out
 
 
-def indexer_scores(ikeys, slot, n_keys, q_idx, w, raw=False):
+INDEXER_GLM, INDEXER_DS = 0, 1
+
+
+def indexer_scores(ikeys, slot, n_keys, q_idx, w, raw=False, mode=None):
     q, qp = _np(q_idx, np.uint16)
     w, wp = _np(w, np.float32)
     ih = q.shape[0]
     out = np.empty(n_keys, np.float32)
-    rc = lib().cwick_hip_indexer_scores(ikeys.h, slot, n_keys, qp, wp, ih, out.ctypes.data)
+    if mode is None:
+        rc = lib().cwick_hip_indexer_scores(ikeys.h, slot, n_keys, qp, wp, ih, out.ctypes.data)
+    else:
+        rc = lib().cwick_hip_indexer_scores_mode(ikeys.h, slot, n_keys, qp, wp, ih, mode,
+                                                 out.ctypes.data)
     if raw:
         return rc, out
     _check(rc, "indexer_scores")

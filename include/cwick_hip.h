@@ -12,7 +12,13 @@
  *     missing device or a HIP error; it never aborts and never approximates.
  *   - cwick_hip_last_error() says why the last call on this thread declined.
  *   - called from the request thread, one generation at a time
- *     (src/attention.c:353-354); calls on one handle must not overlap.
+ *     (src/attention.c:353-354); calls on one handle must not overlap.  Every
+ *     cache handle owns a HIP stream and a staging buffer for the operands of
+ *     its host-pointer calls, so calls on different handles may run on different
+ *     threads (the per-slot model of src/metal.c:306-319).  The two host-pointer
+ *     calls that take no handle (cwick_hip_topk, cwick_hip_e4m3_table) take
+ *     turns under a lock.  The *_dev calls use the caller's stream and a
+ *     split-K workspace per stream: one thread per stream.
  *
  * MI355X has its own memory, so caches live in device memory behind opaque
  * handles that the engine fills at the sites where it writes its host caches
@@ -84,6 +90,11 @@ int cwick_hip_kv_write(cwick_hip_kv *c, int64_t pos0, int64_t n,
  * (q35_narrow_rows, src/q35_model.c:1558-1575). */
 int cwick_hip_kv_write_f32(cwick_hip_kv *c, int64_t pos0, int64_t n,
                            const float *k_rows, const float *v_rows);
+/* Read rows back as stored (bf16), or widened to fp32 on the device
+ * (q35_widen_rows, src/q35_model.c:1543-1556): what a prefix snapshot of the
+ * caches takes (src/pfx.h:42-73, src/engine.c:3630-3660). */
+int cwick_hip_kv_read(cwick_hip_kv *c, int64_t pos0, int64_t n, uint16_t *k_rows, uint16_t *v_rows);
+int cwick_hip_kv_read_f32(cwick_hip_kv *c, int64_t pos0, int64_t n, float *k_rows, float *v_rows);
 uint16_t *cwick_hip_kv_k_dev(cwick_hip_kv *c);   /* device addresses, for */
 uint16_t *cwick_hip_kv_v_dev(cwick_hip_kv *c);   /* callers that fill in HBM */
 
@@ -119,6 +130,9 @@ int cwick_hip_ikeys_write(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
                           const uint8_t *rows, const float *scales);
 int cwick_hip_ikeys_write_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
                               const float *rows);
+/* Read rows back (the indexer pools of a prefix snapshot, src/pfx.h:42-73). */
+int cwick_hip_ikeys_read(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n, uint8_t *rows,
+                         float *scales);
 uint8_t *cwick_hip_ikeys_rows_dev(cwick_hip_ikeys *c, int slot);
 float *cwick_hip_ikeys_scales_dev(cwick_hip_ikeys *c, int slot);
 
@@ -128,8 +142,8 @@ float *cwick_hip_ikeys_scales_dev(cwick_hip_ikeys *c, int slot);
  * dec_out_slices (src/q35_model.c:1656-1701).  One query position, every
  * head: out[h] = softmax_t(scale * q[h].K[t][h/group]) . V[.][h/group] over
  * t in [0, n_keys).  q [n_heads][head_dim] bf16, out [n_heads][head_dim] fp32.
- * Supported: head_dim 256 or 128, n_heads a multiple of n_kv_heads with group
- * <= 8, 1 <= n_keys <= capacity. */
+ * Supported: head_dim 256 or 128, group = n_heads/n_kv_heads in {1,2,4,8},
+ * 1 <= n_keys <= capacity. */
 int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q,
                          int n_heads, float scale, float *out);
 
@@ -154,6 +168,16 @@ int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16
 int cwick_hip_mla_decode(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
                          const uint16_t *q, int n_heads, float scale, float *out);
 
+/* The same with the attention sink of ds_sparse_attn_heads (src/ds_model.c:917-966,
+ * the sink term at :946): sink [n_heads] fp32, in the units of the scaled scores;
+ * exp(sink[h] - max) joins the softmax denominator of head h and carries no
+ * value.  sink == NULL is cwick_hip_mla_decode.  The reference's index list
+ * addresses two stores -- t < W the window ring, else compressed row t - W
+ * (:930-931) -- which here is one slot whose first W rows hold the ring. */
+int cwick_hip_mla_decode_sink(cwick_hip_latent *c, int slot, const int32_t *sel, int64_t n_list,
+                              const uint16_t *q, int n_heads, float scale, const float *sink,
+                              float *out);
+
 /* Replaces the per-token loop of cwick_attention_mla_prefill_chunk
  * (src/attention.c:1010-1019): n queries at positions pos0..pos0+n-1, query t
  * attends rows 0..pos0+t of the slot (npos = pos+1, :662), all of which are
@@ -173,6 +197,20 @@ int cwick_hip_mla_prefill_chunk(cwick_hip_latent *c, int slot, int64_t pos0, int
 int cwick_hip_indexer_scores(cwick_hip_ikeys *c, int slot, int64_t n_keys,
                              const uint16_t *q_idx, const float *w, int n_idx_heads,
                              float *scores);
+
+/* The two CPU score loops differ in their roundings; `mode` picks whose bits
+ * the scores reproduce:
+ *   CWICK_HIP_INDEXER_GLM  indexer_select (src/attention.c:573-582): four-lane
+ *                          dot_f32 order, ReLU, times w[h]; what
+ *                          cwick_hip_indexer_scores computes.
+ *   CWICK_HIP_INDEXER_DS   ds_indexer (src/ds_model.c:1099-1121): serial dot over
+ *                          the dequantised key, the dot rounded to bf16
+ *                          (ds_bf16_round) before the ReLU, w[h] rounded to
+ *                          bf16 (the kernel rounds what it is given). */
+enum { CWICK_HIP_INDEXER_GLM = 0, CWICK_HIP_INDEXER_DS = 1 };
+int cwick_hip_indexer_scores_mode(cwick_hip_ikeys *c, int slot, int64_t n_keys,
+                                  const uint16_t *q_idx, const float *w, int n_idx_heads,
+                                  int mode, float *scores);
 
 /* No counterpart in the reference: the first stage of the fused select
  * (cwick_hip_dsa_decode), on its own, for checking it.  scores[t] approximates
@@ -228,6 +266,12 @@ int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales,
                              const uint16_t *q, int n_heads, float scale, float *out,
                              void *stream);
 
+int cwick_hip_mla_decode_sink_dev(const uint8_t *rows, const float *scales,
+                                  int64_t row_batch_stride, int64_t scale_batch_stride,
+                                  int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
+                                  const uint16_t *q, int n_heads, float scale, const float *sink,
+                                  float *out, void *stream);
+
 int cwick_hip_mla_prefill_chunk_dev(const uint8_t *rows, const float *scales, int64_t pos0,
                                     int64_t n, const uint16_t *q, int n_heads, float scale,
                                     float *out, void *stream);
@@ -237,6 +281,12 @@ int cwick_hip_indexer_scores_dev(const uint8_t *keys, const float *kscale,
                                  int batch, int64_t n_keys, const uint16_t *q_idx,
                                  const float *w, int n_idx_heads, float *scores,
                                  void *stream);
+
+int cwick_hip_indexer_scores_mode_dev(const uint8_t *keys, const float *kscale,
+                                      int64_t key_batch_stride, int64_t kscale_batch_stride,
+                                      int batch, int64_t n_keys, const uint16_t *q_idx,
+                                      const float *w, int n_idx_heads, int mode, float *scores,
+                                      void *stream);
 
 /* scores [batch][n], out_idx [batch][k] (rows padded with -1 past min(k,n)). */
 int cwick_hip_topk_dev(const float *scores, int batch, int64_t n, int64_t k,

@@ -14,32 +14,43 @@
  * the reference algorithm runs on the decoded floats.
  *
  * Pinning status (what independent evidence each function is checked against
- * in tests/):
+ * in tests/).  oracle/_ref is the reference's ds_ops.c, tensor.c, util.c, pool.c
+ * and log.c compiled as they lie; src/attention.c (needs the Metal bridge) and
+ * src/q35_model.c, src/mm_model.c, src/ds_quant.c (NEON only) do not build on
+ * this host, so nothing below is checked against object code of those files.
  *   orc_e4m3_to_f32, orc_e4m3_lut      closed form over all 256 bytes, the two
  *                                      reference decoders against each other,
- *                                      oracle/_ref (tensor.c compiled as is)
+ *                                      oracle/_ref (tensor.c)
  *   orc_f32_to_e4m3                    the reference's encoder as written, lost carry
  *                                      below 2^-6 included (known-answer test)
  *   orc_f32_to_e4m3_rne                nearest-grid-point brute force, idempotence,
  *                                      saturation (tools/ds_verify.c:48-63 property)
  *   orc_bf16_*, orc_f32_to_bf16_*      tests/test_cwick.c:72-83 values, bit recipe,
- *                                      oracle/_ref (util.c, ds_ops.c compiled as is)
+ *                                      oracle/_ref (util.c, ds_ops.c)
  *   orc_softmax                        closed forms, double brute force, oracle/_ref
- *   orc_dot_f32                        oracle/_ref via the reference's own callers
- *   orc_topk_heap                      oracle/_ref (ds_ops.c compiled as is), golden vectors
+ *                                      (cwick_softmax and ds_softmax, bit for bit)
+ *   orc_dot_f32                        a constructed case where the four-lane order
+ *                                      shows, double brute force
+ *   orc_topk_heap                      oracle/_ref (ds_topk_scores), golden vectors,
+ *                                      ties included
  *   orc_topk_contract                  brute-force sort, known answers
- *   orc_topk_quickselect               oracle/_ref (attention.c selector through
- *                                      cwick_attention_mla_decode), brute force
+ *   orc_topk_quickselect               known answers traced by hand through
+ *                                      src/attention.c:529-543 and :585-598 (they
+ *                                      separate the threshold at want-1 from want and
+ *                                      show the under-selection), subset-of-contract
+ *                                      property
  *   orc_gqa_decode / orc_gqa_prefill   double brute force, decode==prefill row,
- *                                      rectangle==triangle; q35_model.c does not
- *                                      compile off aarch64: PARITY UNPINNED against
- *                                      a reference build, pinned by mathematics only
- *   orc_mla_decode                     oracle/_ref (attention.c absorbed-latent path
- *                                      with identity W_k/W_v, bit-exact on fp32
- *                                      latents), un-absorbed identity, brute force
- *   orc_mla_prefill_chunk              loop-of-decodes identity, oracle/_ref
- *   orc_indexer_scores                 brute force in double, oracle/_ref
- *                                      (attention.c indexer through the selector)
+ *                                      rectangle==triangle: PARITY UNPINNED against a
+ *                                      reference build, pinned by mathematics only
+ *   orc_mla_decode[_f32]               double brute force over the dequantised latent,
+ *                                      dense == sel 0..n-1, permutation invariance,
+ *                                      the absorption identity of src/attention.c:838-893:
+ *                                      PARITY UNPINNED against a reference build
+ *   orc_mla_prefill_chunk              loop-of-decodes identity, bit for bit: PARITY
+ *                                      UNPINNED against a reference build
+ *   orc_indexer_scores[_ds]            double brute force, ReLU-before-weight, thread
+ *                                      count invariance: PARITY UNPINNED against a
+ *                                      reference build
  */
 #include <math.h>
 #include <stdint.h>
@@ -626,6 +637,112 @@ ORC_API void orc_indexer_scores(const uint16_t *q_bf16,  /* [ih][hd] */
         free(e);
     }
     free(q);
+}
+
+/* src/ds_model.c:1099-1121 (ds_indexer's score loop) on BASELINE's FP8 keys: the key the
+ * reference holds in fp32 is the dequantised one, e4m3(byte) * kscale[t]; the dot is serial
+ * over i (`d += qh[i] * kt[i]`, :1115), rounded to bf16 (`ds_bf16_round(d)`, :1116), kept when
+ * positive and weighted by iw[h], which is itself rounded to bf16 (:1101; the caller passes
+ * w[h] = weights_proj * IH^-1/2 * NH^-1/2 and the rounding happens here). */
+ORC_API void orc_indexer_scores_ds(const uint16_t *q_bf16,  /* [ih][hd] */
+                                   const float *w,          /* [ih] */
+                                   const uint8_t *keys,     /* [n][hd] e4m3 */
+                                   const float *kscale,     /* [n] */
+                                   int64_t n, int ih, int hd, int nthreads,
+                                   float *sc /* [n] */) {
+    float lut[256];
+    orc_e4m3_lut(lut);
+    nthreads = orc_threads(nthreads);
+    float *q = malloc(sizeof(float) * (size_t)ih * hd);
+    float *iw = malloc(sizeof(float) * (size_t)ih);
+    for (int i = 0; i < ih * hd; i++) q[i] = orc_bf16_to_f32(q_bf16[i]);
+    for (int h = 0; h < ih; h++) iw[h] = orc_bf16_round(w[h]);
+#pragma omp parallel num_threads(nthreads)
+    {
+        float *kt = malloc(sizeof(float) * (size_t)hd);
+#pragma omp for schedule(static)
+        for (int64_t t = 0; t < n; t++) {
+            for (int i = 0; i < hd; i++) kt[i] = lut[keys[t * hd + i]] * kscale[t];
+            float acc = 0.0f;
+            for (int h = 0; h < ih; h++) {
+                const float *qh = q + (size_t)h * hd;
+                float d = 0.0f;
+                for (int i = 0; i < hd; i++) d += qh[i] * kt[i];
+                d = orc_bf16_round(d);
+                if (d > 0.0f) acc += d * iw[h];
+            }
+            sc[t] = acc;
+        }
+        free(kt);
+    }
+    free(iw);
+    free(q);
+}
+
+/* src/ds_model.c:917-966 (ds_sparse_attn_heads) on BASELINE's FP8 latent: per head, scores
+ * over idx[] with a serial dot (`d += qh[i] * kt[i]`, then `d *= scale`, :933-934), entries < 0
+ * skipped, running maximum from -1e30 (:926), float sum of expf(score - max) (:939-944), the
+ * sink term expf(sink[h] - max) added to the sum only (:946), values accumulated in list order
+ * and scaled by 1/sum at the end (:948-958).  The reference's key and value are the same 512
+ * floats (HD); here the score uses kdim, the value the first vdim of the same row, as
+ * orc_mla_decode does.  idx == NULL means 0..nlist-1.  An entry of the reference's list
+ * addresses the window ring below W and compressed row t - W from there (:930-931): one cache
+ * whose first W rows are the ring. */
+ORC_API void orc_sparse_attn_sink(const uint16_t *q_bf16,   /* [nh][kdim] */
+                                  const uint8_t *lat, const float *lat_scales,
+                                  int64_t kdim, int64_t vdim, int64_t block,
+                                  const int32_t *idx, int64_t nlist, int nh, float scale,
+                                  const float *sink /* [nh] or NULL */, int nthreads,
+                                  float *out /* [nh][vdim] */) {
+    float lut[256];
+    orc_e4m3_lut(lut);
+    const int64_t nblk = (kdim + block - 1) / block;
+    nthreads = orc_threads(nthreads);
+    /* the rows are decoded once; the reference's caches hold them decoded */
+    float *rows = malloc(sizeof(float) * (size_t)(nlist > 0 ? nlist : 1) * kdim);
+    for (int64_t j = 0; j < nlist; j++) {
+        const int64_t t = idx ? idx[j] : j;
+        if (t >= 0) latent_row_f32(lat + t * kdim, lat_scales + t * nblk, kdim, block, lut, rows + j * kdim);
+    }
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int h = 0; h < nh; h++) {
+        float *qh = malloc(sizeof(float) * (size_t)kdim);
+        float *sc = malloc(sizeof(float) * (size_t)(nlist > 0 ? nlist : 1));
+        float *oh = out + (size_t)h * vdim;
+        for (int64_t i = 0; i < kdim; i++) qh[i] = orc_bf16_to_f32(q_bf16[(size_t)h * kdim + i]);
+        float mx = -1e30f;
+        for (int64_t j = 0; j < nlist; j++) {
+            const int64_t t = idx ? idx[j] : j;
+            if (t < 0) { sc[j] = -INFINITY; continue; }
+            const float *kt = rows + j * kdim;
+            float d = 0.0f;
+            for (int64_t i = 0; i < kdim; i++) d += qh[i] * kt[i];
+            d *= scale;
+            sc[j] = d;
+            if (d > mx) mx = d;
+        }
+        float sum = 0.0f;
+        for (int64_t j = 0; j < nlist; j++) {
+            const int64_t t = idx ? idx[j] : j;
+            if (t < 0) { sc[j] = 0.0f; continue; }
+            const float e = expf(sc[j] - mx);
+            sc[j] = e;
+            sum += e;
+        }
+        if (sink) sum += expf(sink[h] - mx);
+        for (int64_t i = 0; i < vdim; i++) oh[i] = 0.0f;
+        for (int64_t j = 0; j < nlist; j++) {
+            const int64_t t = idx ? idx[j] : j;
+            if (t < 0) continue;
+            const float *kt = rows + j * kdim;
+            const float wgt = sc[j];
+            for (int64_t i = 0; i < vdim; i++) oh[i] += wgt * kt[i];
+        }
+        const float inv = 1.0f / sum;
+        for (int64_t i = 0; i < vdim; i++) oh[i] *= inv;
+        free(sc); free(qh);
+    }
+    free(rows);
 }
 
 /* ------------------------------------------------------------------ */

@@ -219,6 +219,47 @@ def indexer_scores(q, w, keys, kscale, n=None, nthreads=1):
     return sc
 
 
+def indexer_scores_ds(q, w, keys, kscale, n=None, nthreads=1):
+    """ds_indexer's score loop (src/ds_model.c:1099-1121): serial dot, bf16-rounded dot and weight."""
+    q = np.ascontiguousarray(q, np.uint16)
+    w = np.ascontiguousarray(w, np.float32)
+    keys = np.ascontiguousarray(keys, np.uint8)
+    kscale = np.ascontiguousarray(kscale, np.float32)
+    ih, hd = q.shape
+    n = keys.shape[0] if n is None else n
+    sc = np.empty(n, np.float32)
+    lib().orc_indexer_scores_ds(_p(q, C.c_uint16), _p(w, C.c_float), _p(keys, C.c_uint8),
+                                _p(kscale, C.c_float), C.c_int64(n), ih, hd, nthreads,
+                                _p(sc, C.c_float))
+    return sc
+
+
+def sparse_attn_sink(q, lat, scales, scale, sink=None, sel=None, nlist=None, nthreads=1,
+                     kdim=KDIM, vdim=VDIM, block=BLOCK):
+    """ds_sparse_attn_heads (src/ds_model.c:917-966) over the FP8 latent: sink term in the denominator."""
+    q = np.ascontiguousarray(q, np.uint16)
+    lat = np.ascontiguousarray(lat, np.uint8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    nh = q.shape[0]
+    if sel is not None:
+        sel = np.ascontiguousarray(sel, np.int32)
+        nlist = sel.size if nlist is None else nlist
+        selp = _p(sel, C.c_int32)
+    else:
+        nlist = lat.shape[0] if nlist is None else nlist
+        selp = None
+    sinkp = None
+    if sink is not None:
+        sink = np.ascontiguousarray(sink, np.float32)
+        sinkp = _p(sink, C.c_float)
+    out = np.empty((nh, vdim), np.float32)
+    lib().orc_sparse_attn_sink(_p(q, C.c_uint16), _p(lat, C.c_uint8), _p(scales, C.c_float),
+                               C.c_int64(kdim), C.c_int64(vdim), C.c_int64(block), selp,
+                               C.c_int64(nlist), nh, C.c_float(scale), sinkp, nthreads,
+                               _p(out, C.c_float))
+    return out
+
+
 def topk_contract(sc, k):
     sc = np.ascontiguousarray(sc, np.float32)
     out = np.empty(max(min(k, sc.size), 1), np.int32)

@@ -23,6 +23,10 @@ def orc():
 def hip():
     """The C-ABI library on a live device.  No fallback: a missing library or a
     device that does not come up fails the GPU tests."""
+    # Some tests hold operands in torch tensors.  torch brings its own copy of the HIP runtime;
+    # loaded after the library's it finds no GPU, loaded first the library shares it (the order
+    # bench.py uses).
+    import torch  # noqa: F401
     from cwick_amd import hip as _hip
     _hip.lib()
     assert _hip.ready(), "libcwick_hip.so could not bring the GPU up: " + _hip.last_error()

@@ -414,3 +414,325 @@ def test_dsa_select_degenerate(hip, orc, kind):
         assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
     ik.free()
     lat.free()
+
+
+# ------------------------------------------------------------------ the two prefill configurations at their full shape
+def test_gqa_prefill_full_shape_sampled(hip, orc):
+    """BASELINE config 2 as benchmarked: 8192 tokens, 16/4/256, one launch of 512 workgroups
+    (128 position blocks, cost-ordered grid, 256 key tiles in the longest rows).  The CPU cannot
+    redo 0.55 TFLOP, so rows are sampled: row t of a prefill is the decode at position t (the
+    oracle's decode, 33 MFLOP a row), at the first and last rows, on both sides of every kind of
+    boundary the kernel has (position blocks of 64, the 1024-key switch between its two variants,
+    32-key tiles) and at random places; two whole 128-query tiles, the first and the last, go
+    through the oracle's prefill itself."""
+    say("[case] gqa_prefill full shape 8192")
+    c = synth.cfg2_gqa_prefill()
+    n, nh, nkv, hd = c["n"], c["nh"], c["nkv"], c["hd"]
+    cache = hip.KVCache(n, nkv, hd)
+    cache.write(0, c["k"].reshape(n, -1), c["v"].reshape(n, -1))
+    got = hip.gqa_prefill(cache, 0, c["q"], c["scale"])
+    assert np.isfinite(got).all()
+    g = synth.rng(2024)
+    rows = sorted(set([0, 1, 31, 32, 63, 64, 65, 127, 128, 1023, 1024, 1025, 1087, 1088, 4095, 4096,
+                       8127, 8128, 8190, 8191] + [int(x) for x in g.integers(0, n, 24)]))
+    worst = 0.0
+    for t in rows:
+        ref = orc.gqa_decode(c["q"][t], c["k"][:t + 1], c["v"][:t + 1], c["scale"], nthreads=0)
+        d = np.abs(got[t] - ref).max()
+        worst = max(worst, d)
+        assert d <= 2e-3 and d / np.abs(ref).max() <= 1e-2, "row %d: max-abs %.3e" % (t, d)
+    say("[parity] gqa_prefill 8192: %d sampled rows, worst max-abs %.3e" % (len(rows), worst))
+    for tile in (0, 63):
+        ref = orc.gqa_prefill(c["q"], c["k"], c["v"], 0, c["scale"], tiles=(tile, tile + 1, 1), nthreads=0)
+        sl = slice(128 * tile, 128 * tile + 128)
+        assert_close(got[sl], ref[sl], "gqa_prefill 8192, query tile %d" % tile)
+    cache.free()
+
+
+def test_mla_prefill_chunk_full_shape_sampled(hip, orc):
+    """BASELINE config 4 as benchmarked: 4096 queries appended to 28672 rows, 128 heads, causal
+    over 32768 positions.  Sampled queries (first, last, around the middle and the 64-key tile
+    edges, random ones) against the oracle's chunk prefill restricted to those queries."""
+    say("[case] mla_prefill_chunk full shape 4096 + 28672")
+    c = synth.cfg4_mla_prefill()
+    n, pos0, nh = c["n"], c["pos0"], c["nh"]
+    cache = hip.LatentCache(1, pos0 + n)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_prefill_chunk(cache, 0, pos0, c["q"], c["scale"])
+    cache.free()
+    assert np.isfinite(got).all()
+    g = synth.rng(4044)
+    qs = sorted(set([0, 1, 62, 63, 64, 2047, 2048, 4094, 4095] + [int(x) for x in g.integers(0, n, 5)]))
+    ref = np.zeros((n, nh, synth.VDIM), np.float32)
+    worst = 0.0
+    for t in qs:
+        orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"], queries=(t, t + 1, 1),
+                              nthreads=0, out=ref)
+        d = np.abs(got[t] - ref[t]).max()
+        worst = max(worst, d)
+        assert d <= 2e-3 and d / np.abs(ref[t]).max() <= 1e-2, "query %d: max-abs %.3e" % (t, d)
+    say("[parity] mla_prefill 4096+28672: %d sampled queries, worst max-abs %.3e" % (len(qs), worst))
+
+
+# ------------------------------------------------------------------ cache appends from fp32, read-back
+def test_kv_write_f32_and_read_back(hip, orc):
+    """q35_narrow_rows / q35_widen_rows (src/q35_model.c:1543-1575): fp32 rows narrowed to bf16 on
+    the device with round-to-nearest-even, bit-equal to the numpy and the oracle's recipe
+    (ties, subnormals and large values included); read back as stored and widened."""
+    say("[case] kv write_f32 / read")
+    g = synth.rng(31)
+    n, nkv, hd = 37, 4, 256
+    k = g.standard_normal((n, nkv * hd), dtype=np.float32)
+    v = g.standard_normal((n, nkv * hd), dtype=np.float32) * np.float32(1e3)
+    k[0, :8] = np.array([1.00390625, 1.01171875, -1.00390625, 0.0, -0.0, 1e-40, 3.3e38, 1.0], np.float32)  # ties up/down
+    cache = hip.KVCache(64, nkv, hd)
+    cache.write_f32(0, k, v)
+    cache.write_f32(40, k[:10], v[:10])                   # an append further along
+    kb, vb = cache.read(0, n)
+    assert np.array_equal(kb, synth.f32_to_bf16(k)) and np.array_equal(vb, synth.f32_to_bf16(v))
+    k40, v40 = cache.read(40, 10)
+    assert np.array_equal(k40, kb[:10]) and np.array_equal(v40, vb[:10])
+    L = orc.lib()
+    assert all(int(kb[0, i]) == L.orc_f32_to_bf16_rne(float(k[0, i])) for i in range(8))
+    kf, vf = cache.read_f32(0, n)
+    assert np.array_equal(kf.view(np.uint32), synth.bf16_to_f32(kb).view(np.uint32))
+    assert np.array_equal(vf.view(np.uint32), synth.bf16_to_f32(vb).view(np.uint32))
+    rc = hip.lib().cwick_hip_kv_read(cache.h, 60, 10, kb.ctypes.data, vb.ctypes.data)
+    assert rc == 0 and "capacity" in hip.last_error()
+    # attention over the rows appended this way = the oracle over rows narrowed on the host
+    k[0, 6] = 1.0                                          # keep the scores finite
+    cache.write_f32(0, k[:1], v[:1])
+    kb, vb = cache.read(0, n)
+    q = synth.normal_bf16(g, (16, hd))
+    got = hip.gqa_decode(cache, n, q, 0.0625)
+    ref = orc.gqa_decode(q, synth.f32_to_bf16(k).reshape(n, nkv, hd), synth.f32_to_bf16(v).reshape(n, nkv, hd), 0.0625)
+    assert_close(got, ref, "gqa_decode over rows appended as fp32", strict=False)
+    cache.free()
+
+
+def test_ikeys_write_f32_and_read_back(hip, orc):
+    say("[case] ikeys write_f32 / read")
+    g = synth.rng(32)
+    x = g.standard_normal((200, synth.IDIM), dtype=np.float32)
+    x[3] = 0.0
+    x[4] *= 1e-5
+    c = hip.IndexKeys(2, 256)
+    c.write_f32(1, 10, x)
+    rows, scales = c.read(1, 10, 200)
+    rq, rs = orc.quantize_rows_e4m3(x, synth.IDIM)
+    assert np.array_equal(rows, rq) and np.array_equal(scales.view(np.uint32), rs[:, 0].view(np.uint32))
+    nq, ns = synth.quantize_rows(x, synth.IDIM)
+    assert np.array_equal(nq, rq)
+    # scores over the keys quantised on the device
+    q = synth.normal_bf16(g, (64, synth.IDIM))
+    w = (g.standard_normal(64, dtype=np.float32) / np.float32(np.sqrt(128.0 * 64))).astype(np.float32)
+    c2 = hip.IndexKeys(1, 256)
+    c2.write(0, 0, rows, scales)
+    got = hip.indexer_scores(c2, 0, 200, q, w)
+    ref = orc.indexer_scores(q, w, rq, rs[:, 0], nthreads=0)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    c.free(); c2.free()
+
+
+# ------------------------------------------------------------------ backend selection
+def test_force_off_declines_and_on_again_works(hip, orc):
+    """cwick_hip_force mirrors cwick_metal_force (src/metal.c:60-79): 0 selects the CPU and every
+    compute call declines with its outputs untouched, 1 selects the GPU again.  shutdown frees
+    the internal workspaces; the next call allocates them anew."""
+    say("[case] force(0) / force(1) / shutdown")
+    c = synth.cfg3_mla_decode(700, 16, seed=5)
+    cache = hip.LatentCache(1, 700)
+    cache.write(0, 0, c["rows"], c["scales"])
+    ref = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=0)
+    assert_close(hip.mla_decode(cache, 0, c["q"], c["scale"], n_list=700), ref, "before force(0)")
+    assert hip.force(False) == 0
+    assert not hip.ready()
+    out = np.full((16, synth.VDIM), 7.0, np.float32)
+    q = np.ascontiguousarray(c["q"], np.uint16)
+    rc = hip.lib().cwick_hip_mla_decode(cache.h, 0, None, 700, q.ctypes.data, 16, c["scale"], out.ctypes.data)
+    assert rc == 0 and (out == 7.0).all()
+    assert "not selected" in hip.last_error() or "unavailable" in hip.last_error()
+    rc, _ = hip.topk(np.arange(8, dtype=np.float32), 3, raw=True)
+    assert rc == 0
+    assert hip.force(True) == 0 and hip.ready()
+    assert_close(hip.mla_decode(cache, 0, c["q"], c["scale"], n_list=700), ref, "after force(1)")
+    hip.shutdown()
+    assert hip.ready()
+    assert_close(hip.mla_decode(cache, 0, c["q"], c["scale"], n_list=700), ref, "after shutdown")
+    assert list(hip.topk(np.array([1, 3, 2, 3], np.float32), 2)) == [1, 3]
+    cache.free()
+
+
+def test_two_handles_on_two_threads(hip, orc):
+    """Every handle has its own stream, staging buffer and split-K workspace: calls on different
+    handles from different threads (one request slot each, src/metal.c:306-319) do not disturb
+    one another."""
+    import threading
+    say("[case] two handles, two threads")
+    cs = [synth.cfg3_mla_decode(4000 + 500 * i, 128, seed=60 + i) for i in range(2)]
+    caches = []
+    for c in cs:
+        h = hip.LatentCache(1, c["n_keys"])
+        h.write(0, 0, c["rows"], c["scales"])
+        caches.append(h)
+    refs = [orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=0) for c in cs]
+    errs = [None, None]
+
+    def work(i):
+        try:
+            for _ in range(30):
+                got = hip.mla_decode(caches[i], 0, cs[i]["q"], cs[i]["scale"], n_list=cs[i]["n_keys"])
+                d = np.abs(got - refs[i]).max()
+                if not d <= 2e-3:
+                    errs[i] = "thread %d: max-abs %.3e" % (i, d)
+                    return
+        except Exception as e:      # noqa: BLE001
+            errs[i] = repr(e)
+    th = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    [t.start() for t in th]
+    [t.join() for t in th]
+    assert errs == [None, None], errs
+    for h in caches:
+        h.free()
+
+
+# ------------------------------------------------------------------ MLA decode: more edge cases
+def test_mla_decode_dev_batched_strides(hip, orc):
+    """cwick_hip_mla_decode_dev with a batch of queries that read different caches (batch
+    strides), one of them through a list: the form the fused DSA step and the benchmark call."""
+    import torch
+    say("[case] mla_decode_dev batch strides")
+    B, n_rows, nh = 3, 3000, 128
+    cs = [synth.cfg3_mla_decode(n_rows, nh, seed=80 + b) for b in range(B)]
+    rows = torch.from_numpy(np.stack([c["rows"] for c in cs])).cuda()
+    scales = torch.from_numpy(np.stack([c["scales"] for c in cs])).cuda()
+    q = torch.from_numpy(np.stack([c["q"] for c in cs]).view(np.int16)).cuda()
+    out = torch.empty((B, nh, synth.VDIM), dtype=torch.float32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.mla_decode_dev(rows, scales, n_rows * synth.KDIM, n_rows * synth.NBLK, n_rows, B, None, n_rows,
+                       q, nh, cs[0]["scale"], out, s)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for b in range(B):
+        ref = orc.mla_decode(cs[b]["q"], cs[b]["rows"], cs[b]["scales"], cs[b]["scale"], nthreads=0)
+        assert_close(got[b], ref, "mla_decode_dev dense, batch row %d" % b)
+    g = synth.rng(83)
+    sel = np.stack([np.sort(g.permutation(n_rows)[:1000]) for _ in range(B)]).astype(np.int32)
+    sel[1, 990:] = -1
+    dsel = torch.from_numpy(sel).cuda()
+    hip.mla_decode_dev(rows, scales, n_rows * synth.KDIM, n_rows * synth.NBLK, n_rows, B, dsel, 1000,
+                       q, nh, cs[0]["scale"], out, s)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for b in range(B):
+        ref = orc.mla_decode(cs[b]["q"], cs[b]["rows"], cs[b]["scales"], cs[b]["scale"], sel=sel[b], nthreads=0)
+        assert_close(got[b], ref, "mla_decode_dev sel, batch row %d" % b)
+
+
+@pytest.mark.parametrize("n_keys", [32768, 2500])
+def test_mla_decode_q_outliers(hip, orc, n_keys):
+    """An absorbed query q_abs = W_k^T q has outliers inside its 128-dim blocks.  The kernel
+    splits Q into two E4M3 terms under one power-of-two scale per head and block, so an outlier
+    sets the scale for its 127 neighbours: elements 256 and 4096 times larger than the rest of
+    their block, in every block kind (nope and rope), must still give scores inside tolerance."""
+    say("[case] mla_decode with outliers in Q", n_keys)
+    c = synth.cfg3_mla_decode(n_keys, 128, seed=1700 + n_keys)
+    qf = synth.bf16_to_f32(c["q"]).copy()
+    g = synth.rng(17)
+    for h in range(128):
+        for blk, width in ((0, 128), (2, 128), (4, 64)):
+            i = 128 * blk + int(g.integers(0, width))
+            # the outlier carries little of the score (small factor on a large element would not
+            # be an outlier): scale the rest of the block down instead, keeping the score's size
+            qf[h, 128 * blk:128 * blk + width] *= np.float32(1.0 / (256.0 if h % 2 else 4096.0))
+            qf[h, i] *= np.float32(256.0 if h % 2 else 4096.0) * np.float32(0.25)
+    q = synth.f32_to_bf16(qf)
+    cache = hip.LatentCache(1, n_keys)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_decode(cache, 0, q, c["scale"], n_list=n_keys)
+    ref = orc.mla_decode(q, c["rows"], c["scales"], c["scale"], nthreads=0)
+    assert_close(got, ref, "mla_decode, outliers in Q, %d keys" % n_keys)
+    cache.free()
+
+
+def test_mla_decode_rows_outside_the_list_do_not_leak(hip, orc):
+    """Masked positions of a tile (a ragged end, -1 entries) must contribute nothing whatever the
+    cache holds elsewhere: row 0 is not in the list and holds NaN bytes and a scale 2^40 times
+    the others; a second unlisted row is all NaN bytes."""
+    say("[case] mla_decode: unlisted rows with NaN bytes and huge scales")
+    n_rows, nh = 3000, 128
+    c = synth.cfg3_mla_decode(n_rows, nh, seed=91)
+    rows, scales = c["rows"].copy(), c["scales"].copy()
+    rows[0, ::3] = 0x7F
+    rows[0, 1::3] = 0xFF
+    scales[0] *= np.float32(2.0 ** 40)
+    rows[1234] = 0x7F
+    scales[1234] = np.float32(np.inf)
+    g = synth.rng(92)
+    pool = np.setdiff1d(np.arange(n_rows), [0, 1234])
+    sel = g.choice(pool, size=1000, replace=False).astype(np.int32)
+    sel[[0, 63, 64, 500, 999]] = -1
+    cache = hip.LatentCache(1, n_rows)
+    cache.write(0, 0, rows, scales)
+    got = hip.mla_decode(cache, 0, c["q"], c["scale"], sel=sel)
+    ref = orc.mla_decode(c["q"], rows, scales, c["scale"], sel=sel, nthreads=0)
+    assert_close(got, ref, "mla_decode sel with poisoned unlisted rows")
+    # a ragged dense list that stops before the poisoned row 1234
+    rows[0] = c["rows"][0]; scales[0] = c["scales"][0]
+    cache.write(0, 0, rows[:1], scales[:1])
+    got = hip.mla_decode(cache, 0, c["q"], c["scale"], n_list=1201)
+    ref = orc.mla_decode(c["q"], rows, scales, c["scale"], nlist=1201, nthreads=0)
+    assert_close(got, ref, "mla_decode dense, poisoned row past the end of the list")
+    cache.free()
+
+
+@pytest.mark.parametrize("n_rows,n_sel", [(5000, 2048), (40000, 0), (300, 40)])
+def test_mla_decode_sink(hip, orc, n_rows, n_sel):
+    """The attention sink of ds_sparse_attn_heads (src/ds_model.c:946): exp(sink[h] - max) in the
+    denominator only.  One launch without split-K (short list), one with (merge kernel)."""
+    say("[case] mla_decode with sink", n_rows, n_sel)
+    nh = 128
+    c = synth.cfg3_mla_decode(n_rows, nh, seed=95 + n_rows)
+    g = synth.rng(96)
+    sel = None
+    if n_sel:
+        sel = g.permutation(n_rows)[:n_sel].astype(np.int32)
+        sel[::97] = -1
+    # sinks around the largest score of each head, so that they matter
+    base = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=sel, nthreads=0)
+    sink = (g.standard_normal(nh) * 2.0 + 5.0).astype(np.float32)
+    cache = hip.LatentCache(1, n_rows)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_decode(cache, 0, c["q"], c["scale"], sel=sel, n_list=None if n_sel else n_rows, sink=sink)
+    ref = orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"], sink=sink, sel=sel, nthreads=0)
+    assert_close(got, ref, "mla_decode sink %d rows" % n_rows)
+    assert np.abs(ref - base).max() > 10 * 2e-3 or n_rows > 10000, "the sink does not show in this case"
+    # every entry skipped: zeros, with or without the sink
+    none = hip.mla_decode(cache, 0, c["q"], c["scale"], sel=np.full(70, -1, np.int32), sink=sink)
+    assert np.array_equal(none, np.zeros_like(none))
+    cache.free()
+
+
+# ------------------------------------------------------------------ the DeepSeek indexer flavour
+@pytest.mark.parametrize("n_keys,ih", [(65536, 64), (1000, 32), (257, 7), (1, 64)])
+def test_indexer_scores_ds_mode_bit_exact(hip, orc, n_keys, ih):
+    """ds_indexer's roundings (src/ds_model.c:1099-1121): serial dot over the dequantised key,
+    bf16-rounded dot before the ReLU, bf16-rounded weight: bit for bit."""
+    say("[case] indexer_scores DS mode", n_keys, ih)
+    g = synth.rng(700 + n_keys)
+    keys, ks = synth.index_keys(g, n_keys)
+    q = synth.normal_bf16(g, (ih, synth.IDIM))
+    w = (g.standard_normal(ih, dtype=np.float32) / np.float32(np.sqrt(128.0 * ih))).astype(np.float32)
+    cache = hip.IndexKeys(1, n_keys)
+    cache.write(0, 0, keys, ks)
+    got = hip.indexer_scores(cache, 0, n_keys, q, w, mode=hip.INDEXER_DS)
+    ref = orc.indexer_scores_ds(q, w, keys, ks, nthreads=0)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "DS-mode scores differ in %d of %d places" % ((got != ref).sum(), n_keys)
+    glm = hip.indexer_scores(cache, 0, n_keys, q, w, mode=hip.INDEXER_GLM)
+    assert np.array_equal(glm.view(np.uint32), hip.indexer_scores(cache, 0, n_keys, q, w).view(np.uint32))
+    if n_keys > 100:
+        assert (glm != got).any()
+    rc, _ = hip.indexer_scores(cache, 0, n_keys, q, w, mode=7, raw=True)
+    assert rc == 0 and "mode" in hip.last_error()
+    cache.free()

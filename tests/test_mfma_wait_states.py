@@ -76,3 +76,36 @@ def test_no_valu_write_right_before_an_mfma_reads_it(src):
     assert n_mfma > 0
     assert not bad, "VALU write within two instructions of the MFMA that reads it: %r" % bad[:3]
     assert not early, "MFMA result read before the matrix pipe has written it: %r" % early[:3]
+
+
+LDS_DMA_SOURCES = ["mla_roles.hip", "gqa_prefill.hip"]
+
+
+@pytest.mark.parametrize("src", LDS_DMA_SOURCES)
+def test_m0_belongs_to_the_lds_copies_only(src):
+    """The global -> LDS copies are issued from inline assembly that sets M0 (the LDS address)
+    itself.  M0 is reserved to the compiler and cannot be declared clobbered, so the sources rely
+    on the compiler having no use of M0 of its own in these kernels: on the compiled code, every
+    instruction that names m0 must be the `s_mov_b32 m0, sN` of a copy statement, followed by its
+    `s_nop 0` and its `global_load_lds_*`, and every such load must follow one."""
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        cmd = [B._hipcc()] + B.COMMON + B.PER_FILE.get(src, []) + [
+            "-w", "-S", "--cuda-device-only", os.path.join(B.CSRC, src), "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        ins = []
+        for line in open(out):
+            t = line.split(";")[0].strip()
+            if not t or t.startswith(".") or t.endswith(":"):
+                continue
+            ins.append(t)
+    n_copies = 0
+    for i, t in enumerate(ins):
+        if re.search(r"\bm0\b", t):
+            assert re.match(r"s_mov_b32 m0, s\d+$", t), "compiler-generated use of m0: " + t
+            assert ins[i + 1] == "s_nop 0" and ins[i + 2].startswith("global_load_lds_"), ins[i:i + 3]
+        if t.startswith("global_load_lds_"):
+            n_copies += 1
+            assert ins[i - 2].startswith("s_mov_b32 m0,") and ins[i - 1] == "s_nop 0", ins[i - 2:i + 1]
+    assert n_copies > 0

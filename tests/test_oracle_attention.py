@@ -186,3 +186,99 @@ def test_indexer_scores_vs_brute_force(orc):
     ks2 = ks.copy()
     ks2[10] *= np.float32(4.0)
     assert orc.indexer_scores(q, w, keys, ks2)[10] == np.float32(4.0) * got[10]
+
+
+# ------------------------------------------------------------------ DeepSeek flavours
+def test_sparse_attn_sink_vs_brute_force(orc):
+    """ds_sparse_attn_heads (src/ds_model.c:917-966): the sink joins the denominator and nothing
+    else.  Brute force in double; the closed form for a single key; sink = -inf reduces to the
+    plain sparse decode; -1 entries are skipped; a wrong sign, a sink added to the numerator or
+    a sink scaled like a score would each fail one of these."""
+    n_rows, nh = 400, 12
+    c = synth.cfg3_mla_decode(n_rows, nh, seed=41)
+    lut = orc.e4m3_lut()
+    lat = dequant(c["rows"], c["scales"], lut)
+    g = synth.rng(42)
+    sel = g.permutation(n_rows)[:150].astype(np.int32)
+    sel[[4, 77]] = -1
+    sink = g.standard_normal(nh).astype(np.float32) * 2.0
+    got = orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"], sink=sink, sel=sel)
+    live = sel[sel >= 0]
+    q = f32(c["q"])
+    s = c["scale"] * (q @ lat[live].T)                                 # [nh, n]
+    m = s.max(axis=1, keepdims=True)
+    e = np.exp(s - m)
+    den = e.sum(axis=1) + np.exp(sink.astype(np.float64) - m[:, 0])
+    want = (e @ lat[live][:, :512]) / den[:, None]
+    assert np.abs(got - want).max() < 2e-5
+    # without the sink the denominators differ visibly on this data (the test has teeth)
+    assert np.abs(want - (e @ lat[live][:, :512]) / e.sum(axis=1)[:, None]).max() > 1e-3
+    # sink = -inf: the plain sparse decode
+    no = orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"],
+                              sink=np.full(nh, -np.inf, np.float32), sel=sel)
+    plain = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=sel)
+    assert np.abs(no - plain).max() < 2e-5
+    assert np.array_equal(no, orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"], sel=sel))
+    # one key: out = v / (1 + exp(sink - score))
+    one = orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"], sink=sink,
+                               sel=np.array([7], np.int32))
+    s7 = c["scale"] * (q @ lat[7])
+    assert np.abs(one - lat[7][None, :512] / (1.0 + np.exp(sink - s7))[:, None]).max() < 2e-5
+    # nothing selected: zeros, as `oh[i] = 0` times 1/inf gives (src/ds_model.c:947-958)
+    none = orc.sparse_attn_sink(c["q"], c["rows"], c["scales"], c["scale"], sink=sink,
+                                sel=np.array([-1, -1], np.int32))
+    assert np.array_equal(none, np.zeros_like(none))
+
+
+def test_indexer_scores_ds_roundings(orc):
+    """ds_indexer's loop (src/ds_model.c:1099-1121): the dot is rounded to bf16 before the ReLU,
+    the weight is rounded to bf16, the dot is serial.  Each known answer below separates one of
+    these from the GLM flavour."""
+    hd = 128
+    lut = orc.e4m3_lut()
+    one = int(np.where(lut == 1.0)[0][0]); v1125 = int(np.where(lut == 1.125)[0][0])
+
+    def run(qrow, keyrow, ks, w):
+        q = synth.f32_to_bf16(np.asarray(qrow, np.float32)[None, :])
+        return float(orc.indexer_scores_ds(q, np.array([w], np.float32), np.asarray(keyrow, np.uint8)[None, :],
+                                           np.array([ks], np.float32))[0])
+    # (1) the dot is rounded to bf16: 1.125 * (1 + 2^-8) = 1.12939453125 -> 1.1328125 (145/128)
+    q = np.zeros(hd); q[0] = 1.0
+    k = np.zeros(hd, np.uint8); k[0] = v1125
+    assert run(q, k, 1.0 + 2.0 ** -8, 1.0) == 1.1328125
+    # (2) the weight is rounded to bf16: 1 + 2^-9 rounds to 1 (ties to even), 1 + 3 * 2^-9 to 1 + 2^-7
+    k[0] = one
+    assert run(q, k, 1.0, 1.0 + 2.0 ** -9) == 1.0
+    assert run(q, k, 1.0, 1.0 + 3 * 2.0 ** -9) == 1.0 + 2.0 ** -7
+    # (3) the ReLU comes after the rounding and before the weight: a negative dot contributes nothing
+    q[0] = -1.0
+    assert run(q, k, 1.0, -5.0) == 0.0
+    # (4) serial order: 2^24 + 1 + 1 + 1 + 1 - 2^24 is 0 added one by one (each 1 is lost) and 4 when
+    #     the four partial lanes of dot_f32 are used; the bf16 rounding keeps both exactly
+    q = np.zeros(hd); k = np.zeros(hd, np.uint8)
+    q[0] = 2.0 ** 24; q[1:5] = 1.0; q[5] = -2.0 ** 24
+    k[:6] = one
+    assert run(q, k, 1.0, 1.0) == 0.0
+    glm = float(orc.indexer_scores(synth.f32_to_bf16(np.asarray(q, np.float32)[None, :]), np.array([1.0], np.float32),
+                                   k[None, :], np.array([1.0], np.float32))[0])
+    assert glm != 0.0
+
+
+def test_indexer_scores_ds_vs_brute_force(orc):
+    g = synth.rng(43)
+    n, ih = 500, 32
+    keys, ks = synth.index_keys(g, n)
+    q = synth.normal_bf16(g, (ih, 128))
+    w = (g.standard_normal(ih) / np.sqrt(128.0 * ih)).astype(np.float32)
+    got = orc.indexer_scores_ds(q, w, keys, ks)
+    lut = orc.e4m3_lut().astype(np.float64)
+    kt = lut[keys] * ks.astype(np.float64)[:, None]
+    d = kt @ f32(q).T                                                    # [n, ih]
+    wb = synth.bf16_to_f32(synth.f32_to_bf16(w)).astype(np.float64)
+    want = (np.maximum(d, 0.0) * wb[None, :]).sum(axis=1)
+    # the bf16 rounding of every dot (2^-9 relative) dominates the error
+    bound = (np.abs(d) * np.abs(wb)[None, :]).sum(axis=1) * 2.0 ** -8 + 1e-6
+    assert (np.abs(got - want) <= bound).all()
+    assert np.abs(got - want).max() > 1e-5            # ... and is really there
+    # threads only split the keys
+    assert np.array_equal(got, orc.indexer_scores_ds(q, w, keys, ks, nthreads=0))

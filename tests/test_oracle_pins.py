@@ -191,6 +191,35 @@ def test_topk_known_answers(orc, sc, k, contract, heap):
             assert list(orc.ref_topk_scores(sc, k)) == heap
 
 
+# Known answers of the GLM selector, traced by hand through src/attention.c:529-543
+# (score_select: Hoare partition around v[(lo+hi)>>1], `k <= j -> hi = j`, `k >= i -> lo = i`,
+# else stop) and :588-598 (thr = copy[want-1]; all `> thr` in index order, then `== thr`).
+# State of the copy after every partition round:
+#   [1,5,2,4,3] want 3: pivot 2 -> [3,5,4,2,1] (i 3, j 2, lo = 3); pivot 2 -> same (i 4, j 2, stop);
+#       thr = copy[2] = 4 -> takes 5 and 4 only: the 3 is lost (copy[3] = 2 would take all three)
+#   [5,3,4,1,2] want 3: pivot 4 -> [5,4,3,1,2] (lo = 2); pivot 1 -> [5,4,3,2,1] (hi = 3);
+#       pivot 3 -> same (lo = 3); thr = 3 -> `> 3`: indices 0, 2, then `== 3`: index 1
+#   [3,1,4,1,5] want 2: pivot 4 -> [5,4,1,1,3] (lo = 2); pivot 1 -> [5,4,3,1,1] (hi = 2);
+#       thr = 4 -> index 4, then index 2
+#   [2,2,1,2,3] want 2: pivot 1 -> [2,2,3,2,1] (hi = 3); pivot 2 -> [2,3,2,2,1] (lo = 2);
+#       pivot 2 -> same (hi = 2); thr = copy[1] = 3 -> index 4 alone (the contract: 0 and 4)
+QUICKSELECT_TRACED = [
+    ([1, 5, 2, 4, 3], 3, [1, 3]),
+    ([5, 3, 4, 1, 2], 3, [0, 2, 1]),
+    ([3, 1, 4, 1, 5], 2, [4, 2]),
+    ([2, 2, 1, 2, 3], 2, [4]),
+]
+
+
+@pytest.mark.parametrize("sc,want,traced", QUICKSELECT_TRACED)
+def test_topk_quickselect_hand_traced(orc, sc, want, traced):
+    sc = np.array(sc, np.float32)
+    assert list(orc.topk_quickselect(sc, want)) == traced
+    # reading the threshold one place later (copy[want]) would give the contract's set on the
+    # first and the last case: the traced answers tell the two apart
+    assert set(traced) <= set(int(i) for i in orc.topk_contract(sc, want))
+
+
 def brute_topk(sc, k):
     order = sorted(range(len(sc)), key=lambda i: (-float(sc[i]), i))
     return sorted(order[:min(k, len(sc))])
