@@ -55,7 +55,7 @@ int launch_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64
 int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
                       const uint16_t *q, int n_heads, float scale, const float *sink, float *out,
-                      hipStream_t s);
+                      hipStream_t s, bool fixed_scratch = false);
 int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,
                        const uint16_t *q, int n_heads, float scale, float *out, hipStream_t s);
 int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_bstride,

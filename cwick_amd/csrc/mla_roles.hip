@@ -725,7 +725,27 @@ mla_merge_frag16_kernel(const uint32_t *__restrict__ part_acc, const float *__re
     *(f32x4 *)(out + ((size_t)y * nh + head) * VDIM + 16 * db + 4 * g) = r4;
 }
 
-int run(Params &p, hipStream_t s) {
+// Split-K partials of the entry point that may not allocate (cwick_hip_mla_decode_static_dev):
+// a fixed area in the library's own device image instead of the grow-only workspace.  Host code
+// never uses the array's name as an address: static_scratch() asks the runtime once where the
+// device's copy lives and hands out that pointer.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+static void *static_scratch() {
+    static std::once_flag once;
+    static void *ptr = nullptr;
+    static hipError_t err = hipSuccess;
+    std::call_once(once, [] {
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) ptr = nullptr;
+    });
+    if (!ptr) hip_ok(err != hipSuccess ? err : hipErrorInvalidSymbol, "hipGetSymbolAddress(scratch)");
+    return ptr;
+}
+
+// fixed == true: partials go to the static area, nothing is allocated and no events are created
+int run(Params &p, hipStream_t s, bool fixed = false) {
     static std::once_flag attr_once;
     static hipError_t attr_err = hipSuccess;
     const size_t smem = sizeof(Smem);
@@ -740,18 +760,28 @@ int run(Params &p, hipStream_t s) {
     if (p.n_splits > 1) {
         const size_t acc_b = (size_t)p.nq * p.n_splits * n_hb * HW * VDIM * sizeof(int16_t);
         const size_t ml_b = (size_t)p.nq * p.n_splits * n_hb * HW * 4 * 4 * sizeof(float);
-        char *ws = (char *)workspace(s, acc_b + ml_b);
-        CWICK_REQUIRE(ws, "mla: workspace allocation failed");
+        char *ws;
+        if (fixed) {
+            CWICK_REQUIRE(acc_b + ml_b <= STATIC_SCRATCH_BYTES,
+                          "mla_decode_static: the split-K partials of this call (%zu bytes) exceed the "
+                          "static scratch area (%zu bytes); use cwick_hip_mla_decode_dev",
+                          acc_b + ml_b, STATIC_SCRATCH_BYTES);
+            ws = (char *)static_scratch();
+            if (!ws) return 0;
+        } else {
+            ws = (char *)workspace(s, acc_b + ml_b);
+            CWICK_REQUIRE(ws, "mla: workspace allocation failed");
+        }
         p.part_acc = (uint32_t *)ws;
         p.part_ml = (float *)(ws + acc_b);
     }
     {
-        ProfScope ps(CWICK_HIP_PROF_MLA, s);
+        ProfScope ps(fixed ? -1 : CWICK_HIP_PROF_MLA, s);
         mla_roles_kernel<<<dim3((unsigned)total), THREADS, smem, s>>>(p);
     }
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
-        ProfScope ps(CWICK_HIP_PROF_MLA_MERGE, s);
+        ProfScope ps(fixed ? -1 : CWICK_HIP_PROF_MLA_MERGE, s);
         if (p.n_splits <= 8)
             mla_merge_frag16_kernel<<<dim3(2 * n_hb * 4, p.nq), 64 * 8, 0, s>>>(
                 p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 1);
@@ -777,7 +807,7 @@ int splits_per_cu() {
 int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstride,
                       int64_t scale_bstride, int64_t n_rows, int batch, const int32_t *sel,
                       int64_t n_list, const uint16_t *q, int n_heads, float scale, const float *sink,
-                      float *out, hipStream_t s) {
+                      float *out, hipStream_t s, bool fixed_scratch) {
     CWICK_REQUIRE(rows && scales && q && out, "mla_decode: null pointer");
     CWICK_REQUIRE(batch >= 1 && batch <= 4096, "mla_decode: batch %d", batch);
     CWICK_REQUIRE(n_heads >= 1 && n_heads <= 128, "mla_decode: n_heads %d (1..128)", n_heads);
@@ -804,7 +834,7 @@ int launch_mla_decode(const uint8_t *rows, const float *scales, int64_t row_bstr
     per = ((per + TK - 1) / TK) * TK;
     p.keys_per_split = per;
     p.n_splits = (int)((n_list + per - 1) / per);
-    return run(p, s);
+    return run(p, s, fixed_scratch);
 }
 
 int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n,

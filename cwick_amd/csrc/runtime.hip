@@ -176,7 +176,7 @@ static double g_prof_ms[CWICK_HIP_PROF_COUNT];
 static int64_t g_prof_n[CWICK_HIP_PROF_COUNT];
 
 ProfScope::ProfScope(int w, hipStream_t s) : which(w), stream(s), slot(nullptr) {
-    if (!g_prof_on) return;
+    if (!g_prof_on || w < 0) return;                  // w < 0: a launch that must not create events
     std::lock_guard<std::mutex> lk(g_prof_mu);
     ProfPair *pp = new ProfPair;
     if (!g_prof_free.empty()) {
@@ -619,6 +619,16 @@ int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales, int64_t r
     if (!backend_ready()) return 0;   /* the reason is recorded */
     return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_rows, batch, sel,
                              n_list, q, n_heads, scale, nullptr, out, (hipStream_t)stream);
+}
+
+int cwick_hip_mla_decode_static_dev(const uint8_t *rows, const float *scales, int64_t row_batch_stride,
+                                    int64_t scale_batch_stride, int64_t n_rows, int batch,
+                                    const int32_t *sel, int64_t n_list, const uint16_t *q, int n_heads,
+                                    float scale, float *out, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_mla_decode(rows, scales, row_batch_stride, scale_batch_stride, n_rows, batch, sel,
+                             n_list, q, n_heads, scale, nullptr, out, (hipStream_t)stream, true);
 }
 
 int cwick_hip_mla_decode_sink_dev(const uint8_t *rows, const float *scales, int64_t row_batch_stride,

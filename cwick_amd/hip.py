@@ -72,6 +72,8 @@ SIGNATURES = {
                                          _vp, _vp]),
     "cwick_hip_mla_decode_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
                                         _flt, _vp, _vp]),
+    "cwick_hip_mla_decode_static_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
+                                               _flt, _vp, _vp]),
     "cwick_hip_mla_decode_sink_dev": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp, _int,
                                              _flt, _vp, _vp, _vp]),
     "cwick_hip_mla_prefill_chunk_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _flt, _vp, _vp]),
@@ -426,6 +428,15 @@ def mla_decode_dev(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel,
                                                  scale_bstride, n_rows, batch, _dp(sel), n_list,
                                                  _dp(q), n_heads, scale, _dp(out), stream),
                   "mla_decode_dev")
+
+
+def mla_decode_static_dev(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list, q,
+                          n_heads, scale, out, stream=None, raw=False):
+    """cwick_hip_mla_decode_dev that allocates nothing (fixed scratch inside the library)."""
+    rc = lib().cwick_hip_mla_decode_static_dev(_dp(rows), _dp(scales), row_bstride, scale_bstride,
+                                               n_rows, batch, _dp(sel), n_list, _dp(q), n_heads,
+                                               scale, _dp(out), stream)
+    return rc if raw else _check(rc, "mla_decode_static_dev")
 
 
 def mla_prefill_chunk_dev(rows, scales, pos0, n, q, n_heads, scale, out, stream=None):

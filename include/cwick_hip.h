@@ -266,6 +266,24 @@ int cwick_hip_mla_decode_dev(const uint8_t *rows, const float *scales,
                              const uint16_t *q, int n_heads, float scale, float *out,
                              void *stream);
 
+/* No counterpart in the reference: cwick_hip_mla_decode_dev for callers that
+ * cannot allocate device memory (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc).  Same operands, same kernels, same
+ * result; the split-K partials go to a fixed 16 MiB area inside the library's
+ * device image instead of the grow-only workspace, and no call of this entry
+ * point allocates or frees anything (no phase-timer events either: launches
+ * made here are not timed).  It declines when the partials of the call would
+ * not fit (they take about 34 KB per workgroup: every shape whose one round
+ * of workgroups -- at most one per compute unit -- is 256 or fewer fits, the
+ * five benchmark configurations included).  All calls of this entry point on
+ * a GPU share that area: calls that overlap in time on one GPU, on whatever
+ * streams, race. */
+int cwick_hip_mla_decode_static_dev(const uint8_t *rows, const float *scales,
+                                    int64_t row_batch_stride, int64_t scale_batch_stride,
+                                    int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
+                                    const uint16_t *q, int n_heads, float scale, float *out,
+                                    void *stream);
+
 int cwick_hip_mla_decode_sink_dev(const uint8_t *rows, const float *scales,
                                   int64_t row_batch_stride, int64_t scale_batch_stride,
                                   int64_t n_rows, int batch, const int32_t *sel, int64_t n_list,
