@@ -1,16 +1,21 @@
 #!/usr/bin/env python
 """bench.py -- attention hot path of libcwick_hip.so on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 1,2,3,4,5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 1,2,3,4,5] [--no-cpu] [--no-check]
 
 One JSON line on stdout.  `value` is the headline of BASELINE.json's metric: decode
 attention microseconds per token at 32K context (configs[2]: MLA absorbed-latent decode,
 128 heads, 32768 x 576 FP8-E4M3 latent), measured as wall time over exactly K steps with
 every operand already resident in HBM.  The same line carries the HBM GB/s of that step,
 the 8K causal GQA prefill TFLOP/s (configs[1]) and one entry per other configuration
-under "configs", each with its kernel times (HIP events on the launch stream, inside
-the library) and roofline fraction, and the CPU baseline: the oracle's restatement of
-the reference algorithm timed on this host's cores.
+under "configs", each with
+  * its kernel times (HIP events on the launch stream, inside the library) and roofline
+    fraction against the published peak and against the ceiling measured in this run
+    (a 128-bit grid-stride read, a loop of nothing but matrix instructions),
+  * "checked": sampled rows of the output the timed kernel left, compared with the CPU
+    oracle after the timing,
+  * "cpu_baseline": the oracle's restatement of the reference algorithm timed on this
+    host's cores on a stated sub-sample of the same workload.
 
 A step = one pass of the hot path over one batch of synthetic input (one decode token,
 one prefill chunk, one batch of 8 DSA queries).
@@ -28,9 +33,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0      # dense bf16 / fp16 MFMA, published
-FP32_VALU_PEAK_TFLOPS = 157.3  # fp32 vector, published
+FP8_PEAK_TFLOPS = 5000.0       # dense fp8 MFMA, published
 
 METRIC = "decode attn µs/token + HBM GB/s @32K ctx; prefill attn TFLOP/s @8K (1 GPU)"
+ATOL, RTOL = 2e-3, 1e-2
+CEIL = {}                      # measured ceilings of this run: hbm_GBps, bf16_TFLOPs, fp8_TFLOPs
 
 
 def log(*a):
@@ -45,9 +52,16 @@ def dev(x):
     return torch.from_numpy(x).cuda()
 
 
+def close(got, ref):
+    d = float(np.abs(got - ref).max())
+    m = float(np.abs(ref).max())
+    return bool(np.isfinite(got).all() and d <= ATOL and d <= RTOL * m), d
+
+
 class Timer:
-    """Wall time of K back-to-back steps with device syncs on both sides, then the same K
-    steps again with the library's phase timers on (HIP events around each kernel)."""
+    """Wall time of K back-to-back steps with device syncs on both sides; then the same K steps
+    again, each bracketed by a pair of events on the launch stream (per-step minimum, median and
+    maximum) with the library's phase timers on (HIP events around each kernel)."""
 
     def __init__(self, hip, torch, steps, warmup):
         self.hip, self.torch, self.steps, self.warmup = hip, torch, steps, warmup
@@ -64,24 +78,53 @@ class Timer:
         wall = (time.perf_counter() - t0) / self.steps
         hip.prof_reset()
         hip.prof_enable(True)
-        for _ in range(self.steps):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(self.steps)]
+        for a, b in ev:
+            a.record()
             step()
+            b.record()
         torch.cuda.synchronize()
         hip.prof_enable(False)
-        kern = {k: {"avg_us": 1e3 * ms / n, "launches": n}
+        per = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+        kern = {k: {"avg_us": round(1e3 * ms / n, 3), "launches": n}
                 for k, (ms, n) in hip.prof_read().items() if n}
-        return wall, kern
+        spread = {"min": round(per[0], 2), "median": round(per[len(per) // 2], 2), "max": round(per[-1], 2),
+                  "n": len(per)}
+        return wall, kern, spread
 
 
-def roofline(bound, alg, seconds, peak, unit, traffic=None):
-    """alg: algorithmic bytes (hbm) or flops (mfma/valu) of ONE launch of the kernel."""
+def roofline(bound, alg, seconds, peak, unit, traffic=None, measured=None, note=None):
+    """alg: algorithmic bytes (hbm) or flops (mfma) of ONE launch of the kernel."""
     ach = alg / seconds / (1e9 if unit == "GB/s" else 1e12)
-    return {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": unit,
-            "frac": round(ach / peak, 4), "traffic": traffic}
+    r = {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": unit,
+         "frac": round(ach / peak, 4), "traffic": traffic}
+    if measured:
+        r["measured_ceiling"] = round(measured, 1)
+        r["frac_of_measured"] = round(ach / measured, 4)
+    if note:
+        r["peak_note"] = note
+    return r
+
+
+def cpu_threads(orc):
+    return min(orc.max_threads(), int(os.environ.get("CWICK_CPU_THREADS", "1000")))
+
+
+def timed(orc, fn, budget_s, min_reps=1, max_reps=30):
+    reps, total, best = 0, 0.0, 1e30
+    while (total < budget_s and reps < max_reps) or reps < min_reps:
+        t0 = orc.now_ns()
+        fn()
+        dt = (orc.now_ns() - t0) * 1e-9
+        total += dt
+        best = min(best, dt)
+        reps += 1
+    return total / reps, best, reps
 
 
 # ---------------------------------------------------------------- the five configurations
-def bench_cfg1(hip, synth, T, stream):
+def bench_cfg1(hip, synth, orc, T, stream, a):
     import torch
     c = synth.cfg1_gqa_decode()
     k, v, q = dev(c["k"]), dev(c["v"]), dev(c["q"])
@@ -89,16 +132,27 @@ def bench_cfg1(hip, synth, T, stream):
 
     def step():
         hip.gqa_decode_dev(k, v, c["n_keys"], c["nkv"], c["hd"], q, c["nh"], c["scale"], out, stream)
-    wall, kern = T.run(step)
+    wall, kern, spread = T.run(step)
     alg = 2 * 4096 * 4 * 256 * 2 + 8192 + 16384
     t = kern["gqa_decode_split_kernel"]["avg_us"] * 1e-6
-    return {"workload": "cfg1 GQA decode 16q/4kv/hd256, 4096 keys bf16", "us_per_step": wall * 1e6,
-            "kernels": kern, "alg_bytes": alg, "flops": 4 * 16 * 4096 * 256,
-            "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s"),
-            "wall_GBps": alg / wall / 1e9}, (c, out)
+    r = {"workload": "cfg1 GQA decode 16q/4kv/hd256, 4096 keys bf16", "us_per_step": wall * 1e6,
+         "step_us": spread, "kernels": kern, "alg_bytes": alg, "flops": 4 * 16 * 4096 * 256,
+         "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s", measured=CEIL.get("hbm_GBps")),
+         "wall_GBps": alg / wall / 1e9}
+    if orc:
+        ref = orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"], nthreads=0)
+        r["checked"], r["check_maxabs"] = close(out.cpu().numpy(), ref)
+        r["check"] = "the whole output against the oracle's decode"
+        if not a.no_cpu:
+            th = cpu_threads(orc)
+            mean, best, reps = timed(orc, lambda: orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"], 16, th), 1.0, 5)
+            r["cpu_baseline"] = {"value": round(mean * 1e6, 1), "unit": "us/token", "cores": th, "kind": "port",
+                                 "sample": "%d full decodes (mean; best %.0f us), position-sliced scores, "
+                                           "16 accumulation slices (src/q35_model.c:1656-1701)" % (reps, best * 1e6)}
+    return r
 
 
-def bench_cfg2(hip, synth, T, stream):
+def bench_cfg2(hip, synth, orc, T, stream, a):
     import torch
     c = synth.cfg2_gqa_prefill()
     k, v, q = dev(c["k"]), dev(c["v"]), dev(c["q"])
@@ -106,17 +160,44 @@ def bench_cfg2(hip, synth, T, stream):
 
     def step():
         hip.gqa_prefill_dev(k, v, 0, c["n"], c["nkv"], c["hd"], q, c["nh"], c["scale"], out, stream)
-    wall, kern = T.run(step)
+    wall, kern, spread = T.run(step)
     n = c["n"]
     flops = 4 * c["nh"] * c["hd"] * n * (n + 1) // 2          # causal count
     t = kern["gqa_prefill_kernel"]["avg_us"] * 1e-6
-    return {"workload": "cfg2 GQA causal prefill 8192 tokens 16q/4kv/hd256 bf16",
-            "us_per_step": wall * 1e6, "kernels": kern, "flops": flops,
-            "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
-            "wall_TFLOPs": flops / wall / 1e12}, (c, out)
+    r = {"workload": "cfg2 GQA causal prefill 8192 tokens 16q/4kv/hd256 bf16",
+         "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern, "flops": flops,
+         "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s", measured=CEIL.get("bf16_TFLOPs")),
+         "roofline_median_launch": roofline("mfma", flops, spread["median"] * 1e-6, BF16_PEAK_TFLOPS, "TFLOP/s",
+                                            measured=CEIL.get("bf16_TFLOPs")),
+         "wall_TFLOPs": flops / wall / 1e12}
+    if orc:
+        rows = [0, 63, 64, 1023, 1024, 4097, 8128, 8191]
+        got = out[rows].cpu().numpy()
+        ok, worst = True, 0.0
+        for i, t_ in enumerate(rows):
+            ref = orc.gqa_decode(c["q"][t_], c["k"][:t_ + 1], c["v"][:t_ + 1], c["scale"], nthreads=0)
+            o, d = close(got[i], ref)
+            ok, worst = ok and o, max(worst, d)
+        r["checked"], r["check_maxabs"] = ok, worst
+        r["check"] = "rows %s of the timed output against the oracle's decode at that position" % rows
+        if not a.no_cpu:
+            th = cpu_threads(orc)
+            tiles = [15, 47, 63]
+            t0 = orc.now_ns()
+            for tl in tiles:
+                orc.gqa_prefill(c["q"], c["k"], c["v"], 0, c["scale"], tiles=(tl, tl + 1, 1), nthreads=th)
+            dt = (orc.now_ns() - t0) * 1e-9
+            fl = sum(4 * c["nh"] * c["hd"] * sum(range(128 * tl + 1, 128 * tl + 129)) for tl in tiles)
+            r["cpu_baseline"] = {"value": round(fl / dt / 1e12, 4), "unit": "TFLOP/s (causal count)", "cores": th,
+                                 "kind": "port",
+                                 "sample": "query tiles %s of 64 (128 queries x 16 heads each, %.2f s): "
+                                           "src/q35_model.c:1713-1746 per (head, tile) with its naive GEMM; "
+                                           "the whole prefill would take about %.0f s at this rate"
+                                           % (tiles, dt, flops / (fl / dt))}
+    return r
 
 
-def bench_cfg3(hip, synth, T, stream):
+def bench_cfg3(hip, synth, orc, T, stream, a):
     import torch
     c = synth.cfg3_mla_decode()
     rows, scales, q = dev(c["rows"]), dev(c["scales"]), dev(c["q"])
@@ -125,43 +206,94 @@ def bench_cfg3(hip, synth, T, stream):
     def step():
         hip.mla_decode_dev(rows, scales, 0, 0, c["n_keys"], 1, None, c["n_keys"], q, c["nh"],
                            c["scale"], out, stream)
-    wall, kern = T.run(step)
+    wall, kern, spread = T.run(step)
     alg = 32768 * (576 + 20) + 128 * 576 * 2 + 128 * 512 * 4
     flops = 2 * 128 * 32768 * (576 + 512)
     t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
-    # HBM bytes of one launch of mla_roles_kernel at this geometry (64 key slices): FETCH_SIZE and
-    # WRITE_SIZE of rocprofv3 --pmc, each scaled by what a 256 MiB copy reads on the same counter
-    # (profiles/mla_decode_cfg3_pmc_traffic.txt): 21.00 MB read + 8.91 MB of split-K partials written
-    traffic = 20512 * 1024 + 8704 * 1024
-    return {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
-                        "+ 5 fp32 block scales/token, bf16 q",
-            "us_per_step": wall * 1e6, "kernels": kern, "alg_bytes": alg, "flops": flops,
-            "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s", traffic),
-            "roofline_mfma": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
-            "wall_GBps": alg / wall / 1e9}, (c, out)
+    traffic = profile_traffic("mla_decode_cfg3_pmc_traffic.txt")
+    r = {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
+                     "+ 5 fp32 block scales/token, bf16 q",
+         "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern, "alg_bytes": alg, "flops": flops,
+         "roofline": roofline("hbm", alg, t, HBM_PEAK_GBS, "GB/s", traffic, measured=CEIL.get("hbm_GBps")),
+         "roofline_mfma": roofline(
+             "mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s", measured=CEIL.get("bf16_TFLOPs"),
+             note="algorithmic flops 2*128*32768*(576+512), each counted once, against the dense bf16/fp16 "
+                  "peak: the value product runs on the fp16 matrix core; the score product runs on the "
+                  "FP8 matrix core (published peak %.0f) with Q as two E4M3 terms, i.e. twice the "
+                  "algorithmic score flops at twice the rate" % FP8_PEAK_TFLOPS),
+         "wall_GBps": alg / wall / 1e9}
+    if orc:
+        ref = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=0)
+        r["checked"], r["check_maxabs"] = close(out.cpu().numpy(), ref)
+        r["check"] = "the whole output against the oracle's decode"
+    return r, c
 
 
-def bench_cfg4(hip, synth, T, stream):
+def profile_traffic(name):
+    """HBM bytes per launch of the dominant kernel as the committed rocprofv3 --pmc summary states
+    them (a line `traffic_bytes: N`), or None when the summary does not carry the line."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            if line.startswith("traffic_bytes:"):
+                return int(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def bench_cfg4(hip, synth, orc, T, stream, a):
     import torch
-    c = synth.cfg4_mla_prefill()
-    rows, scales, q = dev(c["rows"]), dev(c["scales"]), dev(c["q"])
-    out = torch.empty((c["n"], c["nh"], 512), dtype=torch.float32, device="cuda")
+    # the cache comes from the host generator; the 604 MB of queries are drawn on the device
+    # (seeded N(0,1), rounded to bf16 with round-to-nearest-even) and only the sampled rows are
+    # copied back for the check
+    n, pos0, nh = 4096, 28672, 128
+    g = synth.rng(synth.SEED0 + 4)
+    rows_h, scales_h = synth.latent_cache(g, pos0 + n)
+    rows, scales = dev(rows_h), dev(scales_h)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(synth.SEED0 + 4)
+    q = torch.randn((n, nh, 576), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    out = torch.empty((n, nh, 512), dtype=torch.float32, device="cuda")
+    scale = float(1.0 / np.sqrt(192.0))
 
     def step():
-        hip.mla_prefill_chunk_dev(rows, scales, c["pos0"], c["n"], q, c["nh"], c["scale"], out, stream)
-    wall, kern = T.run(step)
-    keys = c["n"] * c["pos0"] + c["n"] * (c["n"] + 1) // 2
-    flops = 2 * c["nh"] * (576 + 512) * keys
-    t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
-    return {"workload": "cfg4 MLA chunked prefill, 4096 queries appended to 28672 FP8 latent rows",
-            "us_per_step": wall * 1e6, "kernels": kern, "flops": flops,
-            "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s"),
-            "wall_TFLOPs": flops / wall / 1e12}, (c, out)
+        hip.mla_prefill_chunk_dev(rows, scales, pos0, n, q.data_ptr(), nh, scale, out, stream)
+    wall, kern, spread = T.run(step)
+    keys = n * pos0 + n * (n + 1) // 2
+    flops = 2 * nh * (576 + 512) * keys
+    kname = "mla_prefill_kernel" if "mla_prefill_kernel" in kern else "mla_roles_kernel"
+    t = kern[kname]["avg_us"] * 1e-6
+    r = {"workload": "cfg4 MLA chunked prefill, 4096 queries appended to 28672 FP8 latent rows",
+         "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern, "flops": flops,
+         "roofline": roofline("mfma", flops, t, BF16_PEAK_TFLOPS, "TFLOP/s", measured=CEIL.get("bf16_TFLOPs")),
+         "wall_TFLOPs": flops / wall / 1e12}
+    if orc:
+        qs = [0, 63, 64, 2048, 4095]
+        ok, worst = True, 0.0
+        th = cpu_threads(orc)
+        cpu_t, cpu_fl = 0.0, 0
+        for t_ in qs:
+            qh = q[t_].view(torch.int16).cpu().numpy().view(np.uint16)
+            t0 = orc.now_ns()
+            ref = orc.mla_decode(qh, rows_h, scales_h, scale, nlist=pos0 + t_ + 1, nthreads=th)
+            cpu_t += (orc.now_ns() - t0) * 1e-9
+            cpu_fl += 2 * nh * 1088 * (pos0 + t_ + 1)
+            o, d = close(out[t_].cpu().numpy(), ref)
+            ok, worst = ok and o, max(worst, d)
+        r["checked"], r["check_maxabs"] = ok, worst
+        r["check"] = "queries %s of the timed output against the oracle's decode at that position" % qs
+        if not a.no_cpu:
+            r["cpu_baseline"] = {"value": round(cpu_fl / cpu_t / 1e12, 4), "unit": "TFLOP/s", "cores": th,
+                                 "kind": "port",
+                                 "sample": "%d of the 4096 queries (%.2f s): the per-token loop of "
+                                           "src/attention.c:1010-1019; the whole chunk would take about %.0f s "
+                                           "at this rate" % (len(qs), cpu_t, flops / (cpu_fl / cpu_t))}
+    return r
 
 
-def bench_cfg5(hip, synth, T, stream):
+def bench_cfg5(hip, synth, orc, T, stream, a, shared=False):
     import torch
-    c = synth.cfg5_dsa()
+    c = synth.cfg5_dsa(shared=shared)
     B, N, K = c["batch"], c["n_keys"], c["topk"]
     ik, iks = dev(c["ikeys"]), dev(c["ikscale"])
     rows, scales = dev(c["rows"]), dev(c["scales"])
@@ -169,48 +301,61 @@ def bench_cfg5(hip, synth, T, stream):
     sc = torch.empty((B, N), dtype=torch.float32, device="cuda")
     sel = torch.empty((B, K), dtype=torch.int32, device="cuda")
     out = torch.empty((B, c["nh"], 512), dtype=torch.float32, device="cuda")
+    st = 0 if shared else 1
 
     def step():
-        hip.dsa_decode_dev(ik, iks, N * 128, N, rows, scales, N * 576, N * 5, B, N, qi, w, c["ih"],
-                           K, q, c["nh"], c["scale"], sc, sel, out, stream)
-    wall, kern = T.run(step)
-    idx_bytes = B * N * 132
+        hip.dsa_decode_dev(ik, iks, st * N * 128, st * N, rows, scales, st * N * 576, st * N * 5, B, N, qi, w,
+                           c["ih"], K, q, c["nh"], c["scale"], sc, sel, out, stream)
+    wall, kern, spread = T.run(step)
+    idx_bytes = (1 if shared else B) * N * 132
     idx_flops = B * 2 * c["ih"] * N * 128
     t_idx = kern["indexer kernels"]["avg_us"] * 1e-6
     t_mla = kern["mla_roles_kernel"]["avg_us"] * 1e-6
     mla_flops = B * 2 * 128 * K * 1088
-    return {"workload": "cfg5 DSA decode, 8 independent queries (own caches): indexer 64x128 over "
-                        "65536 FP8 keys -> exact top-2048 -> sparse MLA",
-            "us_per_step": wall * 1e6, "us_per_query": wall * 1e6 / B, "kernels": kern,
-            # the indexer phase of the fused call: approximate scores on the matrix cores (one pass
-            # over the key bytes), the select on them, exact rescoring of the keys in the band
-            "roofline": roofline("hbm", idx_bytes, t_idx, HBM_PEAK_GBS, "GB/s"),
-            "roofline_indexer_mfma": roofline("mfma", idx_flops, t_idx, BF16_PEAK_TFLOPS, "TFLOP/s"),
-            "roofline_sparse_mla_mfma": roofline("mfma", mla_flops, t_mla, BF16_PEAK_TFLOPS, "TFLOP/s"),
-            "alg_bytes_indexer": idx_bytes}, (c, (out, sel))
+    r = {"workload": "cfg5 DSA decode, 8 independent queries (%s): indexer 64x128 over 65536 FP8 keys -> "
+                     "exact top-2048 -> sparse MLA" % ("one shared context" if shared else "own caches"),
+         "us_per_step": wall * 1e6, "us_per_query": wall * 1e6 / B, "step_us": spread, "kernels": kern,
+         # the indexer phase of the fused call: approximate scores on the matrix cores (one pass
+         # over the key bytes), the select on them, exact rescoring of the keys in the band
+         "roofline": roofline("hbm", idx_bytes, t_idx, HBM_PEAK_GBS, "GB/s", measured=CEIL.get("hbm_GBps")),
+         "roofline_indexer_mfma": roofline("mfma", idx_flops, t_idx, BF16_PEAK_TFLOPS, "TFLOP/s"),
+         "roofline_sparse_mla_mfma": roofline("mfma", mla_flops, t_mla, BF16_PEAK_TFLOPS, "TFLOP/s"),
+         "alg_bytes_indexer": idx_bytes}
+    if orc:
+        got_sel, got = sel.cpu().numpy(), out.cpu().numpy()
+        ok, worst, th = True, 0.0, cpu_threads(orc)
+        cpu_t = 0.0
+        for b in (0, B - 1):
+            cb = 0 if shared else b
+            t0 = orc.now_ns()
+            s_ = orc.indexer_scores(c["q_idx"][b], c["w"][b], c["ikeys"][cb], c["ikscale"][cb], nthreads=th)
+            rsel = orc.topk_contract(s_, K)
+            ref = orc.mla_decode(c["q"][b], c["rows"][cb], c["scales"][cb], c["scale"], sel=rsel, nthreads=th)
+            cpu_t += (orc.now_ns() - t0) * 1e-9
+            o, d = close(got[b], ref)
+            ok = ok and o and bool(np.array_equal(got_sel[b], rsel))
+            worst = max(worst, d)
+        r["checked"], r["check_maxabs"] = ok, worst
+        r["check"] = "queries 0 and %d: selected indices bit for bit, outputs against the oracle" % (B - 1)
+        if not a.no_cpu:
+            r["cpu_baseline"] = {"value": round(cpu_t / 2 * 1e6, 1), "unit": "us/query", "cores": th, "kind": "port",
+                                 "sample": "2 of the 8 queries: indexer scores (src/attention.c:573-582), "
+                                           "contract top-k, sparse decode (src/attention.c:749-811)"}
+    return r
 
 
 # ---------------------------------------------------------------- CPU baseline (oracle, "port")
-def cpu_baseline_cfg3(c, budget_s):
+def cpu_baseline_cfg3(orc, c, budget_s):
     """The oracle's restatement of src/attention.c:749-811 over BASELINE's FP8 storage, all
     host cores, bounded to about `budget_s` seconds of work."""
-    from oracle import orc
-    threads = min(orc.max_threads(), int(os.environ.get("CWICK_CPU_THREADS", "1000")))
-    reps, t_total = 0, 0.0
-    best = 1e30
-    while (t_total < budget_s and reps < 30) or reps < 2:
-        t0 = orc.now_ns()
-        orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], nthreads=threads)
-        dt = (orc.now_ns() - t0) * 1e-9
-        t_total += dt
-        best = min(best, dt)
-        reps += 1
-    med = t_total / reps
-    return {"value": round(med * 1e6, 1), "unit": "us/token", "cores": threads, "kind": "port",
+    threads = cpu_threads(orc)
+    mean, best, reps = timed(orc, lambda: orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"],
+                                                         nthreads=threads), budget_s, 2)
+    return {"value": round(mean * 1e6, 1), "unit": "us/token", "cores": threads, "kind": "port",
             "sample": "%d full decodes of the same 32768-key workload (mean; best %.0f us), "
                       "position-sliced scores, head-sliced softmax, %d accumulation slices, "
                       "gcc -O2 -fopenmp, nproc=%d" % (reps, best * 1e6, threads, os.cpu_count()),
-            "GBps": round((32768 * 596 + 147456 + 262144) / med / 1e9, 2)}
+            "GBps": round((32768 * 596 + 147456 + 262144) / mean / 1e9, 2)}
 
 
 def main():
@@ -218,10 +363,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="1,2,3,5",
-                    help="which configurations to time besides the headline (cfg4 takes ~1 min)")
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--configs", default="1,2,3,4,5",
+                    help="which configurations to time besides the headline (3 always runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--no-check", action="store_true", help="skip the output checks (and the CPU baselines)")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the read and matrix-core probes")
+    ap.add_argument("--cpu-seconds", type=float, default=6.0)
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known HBM traffic, "
                          "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -237,6 +384,13 @@ def main():
     if not hip.ready():
         log("bench.py: libcwick_hip.so could not bring the GPU up: " + hip.last_error())
         return 1
+    orc = None
+    if not a.no_check:
+        from oracle import orc as _orc       # the checker and the reported CPU baseline, never the timed path
+        orc = _orc
+        orc.lib()
+    else:
+        a.no_cpu = True
     log("[device]", hip.device_info())
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
@@ -250,27 +404,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if not a.no_ceilings:
+        CEIL["hbm_GBps"] = hip.probe_hbm_read(4 << 30, 5)
+        CEIL["bf16_TFLOPs"] = hip.probe_mfma(0, 3)
+        CEIL["fp8_TFLOPs"] = hip.probe_mfma(1, 3)
+        log("[ceilings] read %.0f GB/s, bf16 MFMA %.0f TFLOP/s, fp8 MFMA %.0f TFLOP/s" %
+            (CEIL["hbm_GBps"], CEIL["bf16_TFLOPs"], CEIL["fp8_TFLOPs"]))
+
     results = {}
     # headline first: exactly K steps of cfg3
     T = Timer(hip, torch, a.steps, a.warmup)
-    r3, (c3, _) = bench_cfg3(hip, synth, T, stream)
+    r3, c3 = bench_cfg3(hip, synth, orc, T, stream, a)
     results["cfg3"] = r3
-    log("[cfg3] %.2f us/token wall, kernel %s" % (r3["us_per_step"], json.dumps(r3["kernels"])))
+    log("[cfg3] %.2f us/token wall, kernel %s, checked %s" % (r3["us_per_step"], json.dumps(r3["kernels"]),
+                                                              r3.get("checked")))
     cpu = None
     if not a.no_cpu:
-        cpu = cpu_baseline_cfg3(c3, a.cpu_seconds)
+        cpu = cpu_baseline_cfg3(orc, c3, a.cpu_seconds)
+        r3["cpu_baseline"] = cpu
         log("[cpu ] %.0f us/token on %d threads" % (cpu["value"], cpu["cores"]))
     del c3
-    side = {1: (bench_cfg1, a.steps), 2: (bench_cfg2, max(3, a.steps // 20)),
+    side = {1: (bench_cfg1, a.steps), 2: (bench_cfg2, max(20, a.steps // 10)),
             4: (bench_cfg4, max(2, a.steps // 100)), 5: (bench_cfg5, max(3, a.steps // 10))}
     for i in sorted(wanted - {3}):
         fn, k = side[i]
-        Ti = Timer(hip, torch, k, max(1, min(a.warmup, k)))
-        r, _ = fn(hip, synth, Ti, stream)
+        Ti = Timer(hip, torch, k, max(1, min(a.warmup, k // 2)))
+        r = fn(hip, synth, orc, Ti, stream, a)
         r["steps"] = k
         results["cfg%d" % i] = r
-        log("[cfg%d] %.2f us/step wall, kernels %s" % (i, r["us_per_step"], json.dumps(r["kernels"])))
+        log("[cfg%d] %.2f us/step wall, kernels %s, checked %s" % (i, r["us_per_step"], json.dumps(r["kernels"]),
+                                                                   r.get("checked")))
         torch.cuda.empty_cache()
+        if i == 5:
+            r = bench_cfg5(hip, synth, orc, Ti, stream, a, shared=True)
+            r["steps"] = k
+            results["cfg5_shared_context"] = r
+            log("[cfg5 shared] %.2f us/step wall, checked %s" % (r["us_per_step"], r.get("checked")))
+            torch.cuda.empty_cache()
 
     line = {
         "metric": METRIC,
@@ -283,12 +453,15 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp8-e4m3 latent, bf16 q; bf16/fp16 MFMA, f32 accumulate",
+        "dtype": "fp8-e4m3 latent, bf16 q; scores on the FP8 MFMA (Q as two E4M3 terms), values on the "
+                 "fp16 MFMA, f32 accumulate (cfg1/cfg2: bf16 MFMA, f32 accumulate)",
         "data": "synthetic",
         "config": {"workload": r3["workload"], "kernel_timing": "HIP events inside the library, "
                    "on the launch stream, second pass of the same K steps"},
         "decode_hbm_GBps_wall": round(r3["wall_GBps"], 1),
         "prefill_TFLOPs_8k": round(results["cfg2"]["wall_TFLOPs"], 1) if "cfg2" in results else None,
+        "checked": all(r.get("checked", False) for r in results.values()) if orc else None,
+        "measured_ceilings": {k: round(v, 1) for k, v in CEIL.items()} or None,
         "roofline": r3["roofline"],
         "roofline_mfma": r3["roofline_mfma"],
         "cpu_baseline": cpu,

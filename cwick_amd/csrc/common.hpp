@@ -119,6 +119,8 @@ int launch_quant_ikeys(const float *rows, int64_t n, uint8_t *out_rows, float *o
 int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s);
 int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
+int run_probe_hbm_read(size_t bytes, int reps, double *gbps);
+int run_probe_mfma(int kind, int reps, double *tflops);
 
 // ---- device helpers ---------------------------------------------------------
 // order-preserving 32-bit key of a score for the radix select: larger score, larger key; NaN

@@ -983,6 +983,18 @@ const char *cwick_hip_prof_name(int which) {
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 
+int cwick_hip_probe_hbm_read(size_t bytes, int reps, double *gbps) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return run_probe_hbm_read(bytes, reps, gbps);
+}
+
+int cwick_hip_probe_mfma(int kind, int reps, double *tflops) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return run_probe_mfma(kind, reps, tflops);
+}
+
 int cwick_hip_e4m3_table(float *out256) {
     clear_error();
     if (!backend_ready()) return 0;   /* the reason is recorded */

@@ -85,6 +85,8 @@ SIGNATURES = {
     "cwick_hip_dsa_decode_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _int, _i64,
                                         _vp, _vp, _int, _i64, _vp, _int, _flt, _vp, _vp, _vp,
                                         _vp]),
+    "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
+    "cwick_hip_probe_mfma": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
     "cwick_hip_prof_enable": (None, [_int]),
     "cwick_hip_prof_reset": (None, []),
@@ -399,6 +401,20 @@ def dsa_decode(ikeys, latent, slot0, slot_step, n_keys, q_idx, w, topk_k, q, sca
         return rc, out, sel
     _check(rc, "dsa_decode")
     return out, sel
+
+
+def probe_hbm_read(nbytes=4 << 30, reps=5):
+    """Measured read ceiling of the device in GB/s (128-bit grid-stride read)."""
+    v = C.c_double(0.0)
+    _check(lib().cwick_hip_probe_hbm_read(nbytes, reps, C.byref(v)), "probe_hbm_read")
+    return v.value
+
+
+def probe_mfma(kind=0, reps=3):
+    """Measured matrix-core ceiling in TFLOP/s: kind 0 bf16 32x32x16, kind 1 FP8 16x16x128."""
+    v = C.c_double(0.0)
+    _check(lib().cwick_hip_probe_mfma(kind, reps, C.byref(v)), "probe_mfma")
+    return v.value
 
 
 def e4m3_table():

@@ -347,6 +347,18 @@ void cwick_hip_prof_reset(void);
 int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches);
 const char *cwick_hip_prof_name(int which);
 
+/* ---- measured ceilings -------------------------------------------------- */
+/* The reference measures what a machine can do before judging a kernel against
+ * it (tools/membwbench.c, tools/gpubw.m; docs/PERF.md:997-1042).  The same two
+ * probes for this device: a 128-bit grid-stride read of `bytes` bytes (take
+ * them well beyond the 256 MB of on-package cache), best of `reps` launches,
+ * in GB/s; and a loop of nothing but matrix instructions on every SIMD, in
+ * TFLOP/s -- kind 0: bf16 32x32x16, kind 1: FP8 (E4M3) 16x16x128, the form
+ * the MLA score stage uses.  Both allocate and free their own buffers and use
+ * the null stream; they are bench.py's, not the engine's. */
+int cwick_hip_probe_hbm_read(size_t bytes, int reps, double *gbps);
+int cwick_hip_probe_mfma(int kind, int reps, double *tflops);
+
 /* Device-side codec check used by the parity tests: decodes all 256 E4M3
  * bytes with the conversion instruction the kernels use into out256 (host). */
 int cwick_hip_e4m3_table(float *out256);
