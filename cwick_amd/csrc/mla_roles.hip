@@ -54,7 +54,6 @@ constexpr int TK = 64;                        // keys per tile
 constexpr int HB = 16;                        // heads per head half (partials are laid out per 16 heads)
 constexpr int HW = 32;                        // heads per workgroup
 constexpr int NST = 4;                        // tile stages
-constexpr int NV = 3;                         // copies per tile a value wave issues (the scoring waves take the rest)
 constexpr int NCOL = KDIM / 16;               // 36 sixteen-byte columns per row
 constexpr int NDB = VDIM / 16;                // 32 sixteen-dim output blocks
 constexpr float LAZY = 4.0f;                  // the reference moves when a tile exceeds it by 2^LAZY
@@ -99,6 +98,8 @@ __device__ __attribute__((aligned(16))) float g_zero_scales[8] = {0.0f};
 struct Tile {
     uint8_t kv[NCOL][TK][16];     // [16-byte column][key][16]     36864 B
     float sc[NBLK][TK];           // [block][key]                   1280 B
+    uint32_t valid[2];            // list kernels: bit k = position k of the tile holds a row
+    uint32_t pad[2];
 };
 struct Xch {                       // what the scoring waves publish per tile
     // fp16 probabilities exp2(s - m), laid out as the B fragments of the value MFMA:
@@ -106,6 +107,7 @@ struct Xch {                       // what the scoring waves publish per tile
     // half is key 8 g + j of that half
     uint32_t p[2][2][4][16][4];
     float m[2][16][4];            // [head half][head][key block]: the reference m they are relative to
+    uint32_t moved[8];            // per scoring wave: its reference for this tile is not the common one
 };
 struct Smem {
     Tile tile[NST];
@@ -136,9 +138,46 @@ __device__ __forceinline__ uint32_t mul_f16x2(uint32_t a, uint32_t b) {
 
 #define LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
+// one instruction per max: the compiler's fmaxf quiets both operands first (a v_max of the
+// operand with itself) because it may not assume they are not signalling NaNs
+__device__ __forceinline__ float vmax(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ uint32_t umax3(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r;
+    asm("v_max3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
+typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+typedef __attribute__((address_space(3))) float lds_f32;
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+// LDS is addressed by byte offsets held in ordinary integers (a generic pointer into LDS costs a
+// null check and a 64-bit add at every use)
+#define LDS_AT(type, a) (*(type *)(size_t)(uint32_t)(a))
+
+// LDS offsets of the parts of Smem
+constexpr uint32_t TILE_B = sizeof(Tile);
+constexpr uint32_t SC_OFF = NCOL * TK * 16;                       // Tile::sc
+constexpr uint32_t VALID_OFF = SC_OFF + NBLK * TK * 4;            // Tile::valid
+constexpr uint32_t X_OFF = NST * TILE_B;                          // Smem::x
+constexpr uint32_t XCH_B = sizeof(Xch);
+constexpr uint32_t XM_OFF = 2 * 2 * 4 * 16 * 4 * 4;               // Xch::m
+constexpr uint32_t XF_OFF = XM_OFF + 2 * 16 * 4 * 4;              // Xch::moved
+
+template <bool SEL>
 __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_void *)smem_raw;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -147,7 +186,6 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     const int kb = wave & 3;         // scoring role: keys 16 kb .. 16 kb + 15 of the tile
     const int hh = (wave >> 2) & 1;  //               heads 16 hh .. 16 hh + 15
     const int cw = wave & 3;         // value role: dims 128 cw .. +127 = scale block cw
-    const int vblk = cw;
     const int n = lane & 15;         // head column / key row of a 16-block / dim row
     const int g = lane >> 4;         // 32-wide contraction block (QK) / 8-wide (PV)
 
@@ -162,22 +200,30 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 
     const uint8_t *rows = p.rows + (size_t)y * p.row_bstride;
     const float *scales = p.scales + (size_t)y * p.scale_bstride;
-    const int32_t *sel = p.sel ? p.sel + (size_t)y * p.n_list : nullptr;
+    const int32_t *sel = SEL ? p.sel + (size_t)y * p.n_list : nullptr;
     const int64_t limit = p.n_list + (int64_t)y * p.list_step;
     const int64_t k_begin = (int64_t)split * p.keys_per_split;
     int64_t k_end = k_begin + p.keys_per_split;
     if (k_end > limit) k_end = limit;
-    const int n_tiles = k_end > k_begin ? (int)((k_end - k_begin + TK - 1) / TK) : 0;
+    const int n_keys = k_end > k_begin ? (int)(k_end - k_begin) : 0;     // of this workgroup
+    const int n_tiles = (n_keys + TK - 1) / TK;
 
-    // copy role: lane = key of the tile
+    // The zero row and its scales: where masked positions of a tile are fetched from.  The
+    // addresses are taken once, here: inside the loops every mention would be a load from the
+    // global offset table.
+    uint64_t zrow = (uint64_t)(uintptr_t)g_zero_row, zsc = (uint64_t)(uintptr_t)g_zero_scales;
+    asm volatile("" : "+s"(zrow), "+s"(zsc));
+
+    // copy role: lane = key of the tile; row of the cache or -1
     auto row_of = [&](int t) -> int {
-        const int64_t i = k_begin + (int64_t)t * TK + lane;
-        int64_t r = -1;
-        if (t < n_tiles && i < k_end) {
-            r = sel ? (int64_t)sel[i] : i;
+        const int i = t * TK + lane;
+        if (!SEL) return (t < n_tiles && i < n_keys) ? (int)(k_begin + i) : -1;    // rows fit 31 bits (checked by the launcher)
+        int r = -1;
+        if (t < n_tiles && i < n_keys) {
+            r = sel[k_begin + i];
             if (r < 0 || r >= p.n_rows) r = -1;
         }
-        return (int)r;
+        return r;
     };
     // global -> LDS copies in assembly: the compiler keeps no account of them, so nothing in the
     // loop waits for the tile in flight except the s_waitcnt before the barrier.  Each statement
@@ -185,34 +231,46 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     // compiler (it cannot be named as clobbered); what keeps this safe is that nothing else in
     // this file makes the compiler use M0, which tests/test_mfma_wait_states.py checks on the
     // compiled code.
-    auto dma16 = [&](const void *gp, const void *lp) {
-        const uint32_t off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void *)lp);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gp), "s"(off) : "memory");
+    auto dma16 = [&](uint64_t gp, uint32_t lds_off) {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gp), "s"(lds_off) : "memory");
     };
-    auto dma4 = [&](const void *gp, const void *lp) {
-        const uint32_t off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void *)lp);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gp), "s"(off) : "memory");
+    auto dma4 = [&](uint64_t gp, uint32_t lds_off) {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gp), "s"(lds_off) : "memory");
     };
-    // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; wave w copies pieces w, w+12, w+24, w+36
-    auto issue = [&](int r, Tile *b) {
-        // masked positions fetch the zero row
-        const uint8_t *gsrc = (r >= 0 ? rows + (int64_t)r * KDIM : g_zero_row) + 16 * wave;
-        dma16(gsrc, &b->kv[wave][0][0]);
-        dma16(gsrc + 192, &b->kv[wave + 12][0][0]);
-        dma16(gsrc + 384, &b->kv[wave + 24][0][0]);
-        if (wave < 5) dma4((r >= 0 ? scales + (int64_t)r * NBLK : g_zero_scales) + wave, &b->sc[wave][0]);
+    // pieces 0..35 = sixteen-byte columns of the 64 rows, 36..40 = scale blocks
+    auto piece = [&](int pc, uint64_t rowp, uint64_t scp, uint32_t tile_off) {
+        if (pc < NCOL) dma16(rowp + 16 * pc, tile_off + pc * (TK * 16));
+        else if (pc < NCOL + NBLK) dma4(scp + 4 * (pc - NCOL), tile_off + SC_OFF + (pc - NCOL) * (TK * 4));
     };
-
-    // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks
-    auto piece = [&](int pc, int r, Tile *b) {
-        if (pc < NCOL) dma16((r >= 0 ? rows + (int64_t)r * KDIM : g_zero_row) + 16 * pc, &b->kv[pc][0][0]);
-        else if (pc < NCOL + NBLK)
-            dma4((r >= 0 ? scales + (int64_t)r * NBLK : g_zero_scales) + (pc - NCOL), &b->sc[pc - NCOL][0]);
+    auto row_ptr = [&](int r) -> uint64_t { return r >= 0 ? (uint64_t)(uintptr_t)rows + (uint64_t)(uint32_t)r * KDIM : zrow; };
+    auto sc_ptr = [&](int r) -> uint64_t { return r >= 0 ? (uint64_t)(uintptr_t)scales + (uint64_t)(uint32_t)r * (NBLK * 4) : zsc; };
+    // this wave's share of a tile: three columns, and a scale block for the first five waves
+    // which of the 64 positions of the tile hold a row (the scoring waves mask the others)
+    auto mark = [&](int r, uint32_t tile_off) {
+        const uint64_t v = __ballot(r >= 0);
+        LDS_AT(lds_u32x2, tile_off + VALID_OFF) = (u32x2){(uint32_t)v, (uint32_t)(v >> 32)};
     };
-    // Only tile 0 is fetched before the loop, by everybody.  In step -1, while tile 0 is scored,
-    // the value waves (nothing to accumulate yet) fetch tile 1, and the scoring waves fetch tile 2
-    // at the end of their step; from step 0 on tile t+3 is fetched during step t.
-    if (n_tiles > 0) issue(row_of(0), &sm.tile[0]);
+    auto share = [&](int r, uint32_t tile_off) {
+        const uint64_t rp = row_ptr(r), sp = sc_ptr(r);
+        piece(wave, rp, sp, tile_off);
+        piece(wave + 12, rp, sp, tile_off);
+        piece(wave + 24, rp, sp, tile_off);
+        if (wave < NBLK) piece(NCOL + wave, rp, sp, tile_off);
+        if (SEL && wave == 0) mark(r, tile_off);
+    };
+    auto whole = [&](int r, uint32_t tile_off) {
+        const uint64_t rp = row_ptr(r), sp = sc_ptr(r);
+#pragma unroll
+        for (int pc = 0; pc < NCOL + NBLK; pc++) piece(pc, rp, sp, tile_off);
+        if (SEL) mark(r, tile_off);
+    };
+    // Tile 0 is fetched by everybody at once; then waves 10 and 11, which have no part in the
+    // preparation of Q, fetch tiles 1 and 2.  From step 0 on tile t+3 is fetched during step t,
+    // every wave its share.
+    if (n_tiles > 0) share(row_of(0), lds0);
+    const bool fetched_whole = (wave == 10 && n_tiles > 1) || (wave == 11 && n_tiles > 2);
+    if (wave == 10 && n_tiles > 1) whole(row_of(1), lds0 + TILE_B);
+    if (wave == 11 && n_tiles > 2) whole(row_of(2), lds0 + 2 * TILE_B);
 
     // ---- Q for 2 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
     // 128-dim block (the hardware pairs the scale of lane (n, g) with k-elements that live in other
@@ -220,7 +278,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     // lane (n, g) holds head n of the half, dims 128 b + 32 g + [0, 32); the rope block is one
     // register set: lanes g < 2 hold the hi term of dims 512 + 32 g.., lanes g >= 2 the lo term of
     // dims 512 + 32 (g - 2).. (the key side repeats its bytes).  Unit u = 5 hhu + b is prepared
-    // by wave u and parked in the third tile stage and the exchange area (neither in use yet).
+    // by wave u and parked in the last tile stage and the exchange area (neither in use yet).
     {
         QPark *park = reinterpret_cast<QPark *>(&sm.tile[NST - 1]);
         if (wave < 10) {
@@ -267,19 +325,18 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 qp->lo[d][lane] = wl;
             }
             qp->sc[lane] = 127 + s;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tile 0 has landed (this wave's share)
+        } else if (fetched_whole) {
+            // the share of tile 0 was issued before the 41 copies of tile 1 or 2, which stay in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NCOL + NBLK) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tile 0 has landed (this wave's share)
         LDS_BARRIER();
     }
 
     const float c0 = p.scale * 1.44269504088896340736f;   // scores in log2 units
     float m_ref[2] = {-INFINITY, -INFINITY};          // of head 16 h2 + n; every wave tracks the same values
-    float l_priv = 0.0f, l_pend = 0.0f;               // scoring role: sum over this lane's keys (head 16 hh + n), relative to m_ref / to the tile's m_loc
-
-    // transpose-read addressing for V^T: lane i of 16-lane group g supplies key kappa(g, i>>1),
-    // bytes 8 (i & 1) .. +7 of the sixteen-byte column
-    const int tr_key = 8 * g + (n >> 1);
-    const int tr_off = (8 * cw) * (TK * 16) + tr_key * 16 + 8 * (n & 1);
 
     if (scorer) {
         i32x8 qhi[4], qlo[4], qrope;
@@ -295,56 +352,71 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             }
             qsc0 |= qp->sc[lane] << (8 * b);
         }
-        const QPark *qp = park + 5 * hh + 4;
+        {
+            const QPark *qp = park + 5 * hh + 4;
 #pragma unroll
-        for (int d = 0; d < 8; d++) qrope[d] = qp->hi[d][lane];
-        qsc1 = qp->sc[lane];
-
+            for (int d = 0; d < 8; d++) qrope[d] = qp->hi[d][lane];
+            qsc1 = qp->sc[lane];
+        }
         LDS_BARRIER();                                // before copies or weights land in the park area
-        // step t: waves 0..7 score tile t+1 (if any), waves 8..11 accumulate tile t (if any).
         // Nothing the compiler has in flight may cross into the loop: its waits would also wait
         // for the copies.
         asm volatile("" : "+v"(qhi[0]), "+v"(qhi[1]), "+v"(qhi[2]), "+v"(qhi[3]), "+v"(qlo[0]), "+v"(qlo[1]), "+v"(qlo[2]), "+v"(qlo[3]), "+v"(qrope), "+v"(qsc0), "+v"(qsc1));
-        int row_nxt = row_of(0);
+
+        float l_priv = 0.0f, l_pend = 0.0f;               // sum over this lane's keys (head 16 hh + n), relative to m_ref / to the tile's m_loc
+        float mr = -INFINITY;                             // m_ref of this wave's head half
+        // per-lane LDS offsets inside a tile: K fragment (key 16 kb + n, columns 8 b + 2 g and the
+        // next), the rope block's (columns 32 + 2 (g & 1)), this lane's four keys' scales
+        const uint32_t k_off = (uint32_t)((2 * g) * (TK * 16) + (16 * kb + n) * 16);
+        const uint32_t kr_off = (uint32_t)((32 + 2 * (g & 1)) * (TK * 16) + (16 * kb + n) * 16);
+        const uint32_t s_off = SC_OFF + (uint32_t)((16 * kb + 4 * g) * 4);
+        // where this lane's four probabilities go: keys 16 (kb & 1) + 4 g + i of half kb >> 1
+        const uint32_t xp_off = (uint32_t)(((((hh * 2 + (kb >> 1)) * 4 + 2 * (kb & 1) + (g >> 1)) * 16 + n) * 4 + 2 * (g & 1)) * 4);
+        const uint32_t xm_off = XM_OFF + (uint32_t)(((hh * 16 + n) * 4 + kb) * 4);
+        const uint32_t xmr_off = XM_OFF + (uint32_t)((hh * 16 + n) * 4 * 4);
+        const uint32_t xf_off = XF_OFF + (uint32_t)(wave * 4);
+        const int tail_tile = n_tiles - 1;
+        const bool ragged = (n_keys & (TK - 1)) != 0;
+
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
-            const int row_now = row_nxt;              // rows of tile t+1, fetched one step ahead
-            row_nxt = row_of(t + 2);
-            const bool do_copy = t + 3 < n_tiles;
-            const int row_cp = do_copy ? row_of(t + 3) : -1;
+            const uint32_t xb = lds0 + X_OFF + (uint32_t)(t & 1) * XCH_B;         // exchange area of tile t
+            const bool do_copy = t >= 0 && t + 3 < n_tiles;
+            const int r_cp = do_copy ? row_of(t + 3) : -1;    // fetched here (a list entry is a load), used at the end of the step
             if (t >= 0) {
-                // what the four key blocks of tile t used as reference for this half's heads
-                const f32x4 ml = *(const f32x4 *)&sm.x[t & 1].m[hh][n][0];
-                const float mr = hh ? m_ref[1] : m_ref[0];
-                const float m_new = fmaxf(mr, fmaxf(fmaxf(ml[0], ml[1]), fmaxf(ml[2], ml[3])));
-                if (__any(m_new != mr || ml[0] != m_new || ml[1] != m_new || ml[2] != m_new || ml[3] != m_new)) {
+                // did any scoring wave move its reference in tile t?  (rare after the first tiles)
+                const u32x4 f0 = LDS_AT(lds_u32x4, xb + XF_OFF), f1 = LDS_AT(lds_u32x4, xb + XF_OFF + 16);
+                const uint32_t any_moved = (f0[0] | f0[1] | f0[2] | f0[3]) | (f1[0] | f1[1] | f1[2] | f1[3]);
+                if (__builtin_amdgcn_readfirstlane(any_moved) != 0u) {
+                    const f32x4 ml = LDS_AT(lds_f32x4, xb + xmr_off);
+                    const float m_new = fmaxf(mr, fmaxf(fmaxf(ml[0], ml[1]), fmaxf(ml[2], ml[3])));
                     const float mo = kb == 0 ? ml[0] : kb == 1 ? ml[1] : kb == 2 ? ml[2] : ml[3];
                     const float fo = mo == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mo - m_new);
                     const float c = mr == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mr - m_new);
                     l_priv = l_priv * c + fo * l_pend;
-                    if (hh) m_ref[1] = m_new; else m_ref[0] = m_new;
+                    mr = m_new;
                 } else {
                     l_priv += l_pend;
                 }
             }
             if (t + 1 < n_tiles) {
                 // ---- scores S^T[key][head] for keys 16 kb.., heads 16 hh.. of tile t+1 ----
-                const Tile &T = sm.tile[(t + 1) % NST];
-                Xch &X = sm.x[(t + 1) & 1];
-                const uint64_t valid = __ballot(row_now >= 0);
+                const uint32_t tb = lds0 + (uint32_t)((t + 1) & (NST - 1)) * TILE_B;
+                const uint32_t xn = lds0 + X_OFF + (uint32_t)((t + 1) & 1) * XCH_B;
+                const uint32_t ka = tb + k_off, kr = tb + kr_off, sa = tb + s_off;
                 auto kfrag = [&](int b) -> i32x8 {
-                    const int col = b < 4 ? 8 * b + 2 * g : 32 + 2 * (g & 1);
-                    const u32x4 k0 = *(const u32x4 *)&T.kv[col][16 * kb + n][0];
-                    const u32x4 k1 = *(const u32x4 *)&T.kv[col + 1][16 * kb + n][0];
+                    const uint32_t a = b < 4 ? ka + (uint32_t)(8 * b) * (TK * 16) : kr;
+                    const u32x4 k0 = LDS_AT(lds_u32x4, a);
+                    const u32x4 k1 = LDS_AT(lds_u32x4, a + TK * 16);
                     return (i32x8){(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
                 };
                 const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
-                f32x4 S = z4;
+                f32x4 S;
                 i32x8 kA = kfrag(0);
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     const i32x8 kN = kfrag(b + 1);
-                    const f32x4 scb = *(const f32x4 *)&T.sc[b][16 * kb + 4 * g];
+                    const f32x4 scb = LDS_AT(lds_f32x4, sa + (uint32_t)b * (TK * 4));
                     f32x4 acc;
                     if (b == 0) {
                         acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
@@ -359,25 +431,38 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                         acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
                         acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
                     }
-                    S += acc * scb;
+                    if (b == 0) S = acc * scb;
+                    else S += acc * scb;
                     kA = kN;
                 }
                 {
-                    const f32x4 scb = *(const f32x4 *)&T.sc[4][16 * kb + 4 * g];
+                    const f32x4 scb = LDS_AT(lds_f32x4, sa + 4u * (TK * 4));
                     const f32x4 acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qrope, z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc1);
                     S += acc * scb;
                 }
                 S *= c0;
-                if (valid != ~0ull) {
-                    const uint32_t bits = (uint32_t)(valid >> (16 * kb)) >> (4 * g);
+                // masked positions: past the end of the list (only the last tile of a dense list),
+                // or entries of sel[] that name no row
+                if (SEL ? true : (ragged && t + 1 == tail_tile)) {
+                    uint64_t valid;
+                    if (SEL) {
+                        const u32x2 vw = LDS_AT(lds_u32x2, tb + VALID_OFF);
+                        valid = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)vw[0]) |
+                                ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)vw[1]) << 32);
+                    } else {
+                        valid = __ballot(row_of(t + 1) >= 0);
+                    }
+                    if (valid != ~0ull) {
+                        const uint32_t bits = (uint32_t)(valid >> (16 * kb)) >> (4 * g);
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        if (!((bits >> i) & 1u)) S[i] = -INFINITY;
+                        for (int i = 0; i < 4; i++)
+                            if (!((bits >> i) & 1u)) S[i] = -INFINITY;
+                    }
                 }
-                float lmax = fmaxf(fmaxf(S[0], S[1]), fmaxf(S[2], S[3]));
-                const float mr = hh ? m_ref[1] : m_ref[0];
+                float lmax = vmax3(S[0], S[1], vmax(S[2], S[3]));
                 float m_loc = mr;
-                if (__any(lmax > mr + LAZY)) {            // rare after the first tiles: only then the lanes of a head confer
+                const bool moves = __any(lmax > mr + LAZY);   // rare after the first tiles: only then the lanes of a head confer
+                if (moves) {
                     lmax = fmaxf(lmax, __shfl_xor(lmax, 16, 64));
                     lmax = fmaxf(lmax, __shfl_xor(lmax, 32, 64));
                     m_loc = lmax > mr + LAZY ? lmax : mr;
@@ -391,23 +476,17 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                     u32x2 d;
                     d[0] = pack_f16_rne(P[0], P[1]);
                     d[1] = pack_f16_rne(P[2], P[3]);
-                    *(u32x2 *)&X.p[hh][kb >> 1][2 * (kb & 1) + (g >> 1)][n][2 * (g & 1)] = d;   // keys 16 (kb & 1) + 4 g + i of the half
+                    LDS_AT(lds_u32x2, xn + xp_off) = d;
                 }
-                if (g == 0) X.m[hh][n][kb] = m_loc;
+                // the reference this key block used (the four lanes of a head write the same word)
+                // and whether it differs from the one every wave holds
+                LDS_AT(lds_f32, xn + xm_off) = m_loc;
+                LDS_AT(lds_u32, xn + xf_off) = moves ? 1u : 0u;
             }
             // the copies this wave issued a step ago (its share of tile t+2) have long landed; its
             // share of tile t+3 goes out now, when the wave would otherwise wait at the barrier
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            if (do_copy) {
-                const int rc = row_cp;
-                if (t >= 0) {
-#pragma unroll
-                    for (int i = 0; i < (NCOL + NBLK - 4 * NV + 7) / 8; i++) piece(4 * NV + wave + 8 * i, rc, &sm.tile[(t + 3) % NST]);
-                } else {                              // all of tile 2
-#pragma unroll
-                    for (int i = 0; i < (NCOL + NBLK + 7) / 8; i++) piece(wave + 8 * i, rc, &sm.tile[2]);
-                }
-            }
+            if (do_copy) share(r_cp, lds0 + (uint32_t)((t + 3) & (NST - 1)) * TILE_B);
             LDS_BARRIER();
         }
 
@@ -425,65 +504,72 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 #pragma unroll
             for (int j = 0; j < 8; j++) oacc[h2][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
         int e_run = E_NONE;                               // 2^e_run is above every scale of this wave's block seen so far
+        uint32_t thr_bits = 0u;                           // bits of 2^e_run: a scale whose bits reach them does not fit
+        float wfac = 0.0f;                                // 2^(WEXP - e_run)
         // the value wave shares its SIMD with two scoring waves that stream MFMAs: without priority
         // its many short VALU instructions wait behind them and it becomes the long pole of the step
         __builtin_amdgcn_s_setprio(3);
-        // pieces 0..35 = sixteen-byte columns, 36..40 = scale blocks; in the loop only the value
-        // waves copy (the scoring waves are the long pole of a step, and a wave that issues copies
-        // stalls while the memory pipeline takes them): wave cw takes pieces cw, cw + 4, ...
-        auto issue_value = [&](int r, Tile *b) {
-#pragma unroll
-            for (int i = 0; i < NV; i++) piece(cw + 4 * i, r, b);
-        };
+        // transpose-read addressing for V^T: lane i of 16-lane group g supplies key 8 g + (i >> 1),
+        // bytes 8 (i & 1) .. +7 of the sixteen-byte column
+        const uint32_t tr_off = (uint32_t)((8 * cw) * (TK * 16) + (8 * g + (n >> 1)) * 16 + 8 * (n & 1));
+        // scales of this wave's block for the keys of this lane's contraction slots (8 g .. +7 of each half)
+        const uint32_t sv_off = SC_OFF + (uint32_t)(cw * (TK * 4) + (8 * g) * 4);
+        // the probabilities of this lane's slots: [head half][key half][g][n][4 dwords]
+        const uint32_t pw_off = (uint32_t)((g * 16 + n) * 16);
+        const uint32_t xml_off = XM_OFF + (uint32_t)(n * 16);
         asm volatile("" ::: "memory");
+        int r_cp = row_of(3);                             // rows of the tile copied in step 0; a list entry is a load: fetched a step ahead
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
             const bool do_copy = t >= 0 && t + 3 < n_tiles;
-            if (do_copy) issue_value(row_of(t + 3), &sm.tile[(t + 3) % NST]);   // the stage tile t-1 left at the last barrier
-            if (t < 0 && n_tiles > 1) {                   // all of tile 1
-                const int r = row_of(1);
-#pragma unroll
-                for (int i = 0; i < (NCOL + NBLK + 3) / 4; i++) piece(cw + 4 * i, r, &sm.tile[1]);
+            if (do_copy) {
+                share(r_cp, lds0 + (uint32_t)((t + 3) & (NST - 1)) * TILE_B);   // the stage tile t-1 left at the last barrier
+                r_cp = row_of(t + 4);
             }
             if (t >= 0) {
                 // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 32 heads, tile t ----
-                const Tile &T = sm.tile[t % NST];
-                const Xch &X = sm.x[t & 1];
-                const uint8_t *vbase = &T.kv[0][0][0] + tr_off;
-                // scales of this wave's block for the keys of this lane's contraction slots
+                const uint32_t tb = lds0 + (uint32_t)(t & (NST - 1)) * TILE_B;
+                const uint32_t xb = lds0 + X_OFF + (uint32_t)(t & 1) * XCH_B;
                 f32x4 sv[2][2];
 #pragma unroll
                 for (int kh = 0; kh < 2; kh++)
 #pragma unroll
-                    for (int q = 0; q < 2; q++) sv[kh][q] = *(const f32x4 *)&T.sc[vblk][32 * kh + 8 * g + 4 * q];
+                    for (int q = 0; q < 2; q++) sv[kh][q] = LDS_AT(lds_f32x4, tb + sv_off + (uint32_t)(kh * 128 + q * 16));
                 u32x4 pw[2][2];                           // [head half][key half]
-                f32x4 ml[2];
 #pragma unroll
-                for (int h2 = 0; h2 < 2; h2++) {
+                for (int h2 = 0; h2 < 2; h2++)
 #pragma unroll
-                    for (int kh = 0; kh < 2; kh++) pw[h2][kh] = *(const u32x4 *)&X.p[h2][kh][g][n][0];
-                    ml[h2] = *(const f32x4 *)&X.m[h2][n][0];
-                }
+                    for (int kh = 0; kh < 2; kh++) pw[h2][kh] = LDS_AT(lds_u32x4, xb + pw_off + (uint32_t)((h2 * 2 + kh) * 1024));
+                const u32x4 f0 = LDS_AT(lds_u32x4, xb + XF_OFF), f1 = LDS_AT(lds_u32x4, xb + XF_OFF + 16);
                 // normaliser of the fp16 weights: a power of two above every scale seen so far (it
-                // only grows, and only then the lanes confer)
+                // only grows, and only then the lanes confer).  Scales are compared as integers:
+                // they are positive, and a negative or NaN scale has the larger bit pattern too.
                 float ecorr = 1.0f;
                 {
-                    float smax = fmaxf(fmaxf(fmaxf(sv[0][0][0], sv[0][0][1]), fmaxf(sv[0][0][2], sv[0][0][3])),
-                                       fmaxf(fmaxf(sv[0][1][0], sv[0][1][1]), fmaxf(sv[0][1][2], sv[0][1][3])));
-                    smax = fmaxf(smax, fmaxf(fmaxf(fmaxf(sv[1][0][0], sv[1][0][1]), fmaxf(sv[1][0][2], sv[1][0][3])),
-                                             fmaxf(fmaxf(sv[1][1][0], sv[1][1][1]), fmaxf(sv[1][1][2], sv[1][1][3]))));
-                    const float thr = e_run == E_NONE ? 0.0f : pow2i(e_run);   // scales below 2^e_run fit
-                    if (__any(smax >= thr && smax > 0.0f)) {
+                    uint32_t sb[16];
 #pragma unroll
-                        for (int o = 32; o > 0; o >>= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
-                        const int e_tile = (int)((__builtin_bit_cast(uint32_t, smax) >> 23) & 0xFFu) - 126;
+                    for (int kh = 0; kh < 2; kh++)
+#pragma unroll
+                        for (int q = 0; q < 2; q++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++) sb[(kh * 2 + q) * 4 + i] = __builtin_bit_cast(uint32_t, sv[kh][q][i]) & 0x7FFFFFFFu;
+                    uint32_t smax = umax3(sb[0], sb[1], sb[2]);
+#pragma unroll
+                    for (int i = 3; i < 15; i += 2) smax = umax3(smax, sb[i], sb[i + 1]);
+                    smax = smax > sb[15] ? smax : sb[15];
+                    if (__any(smax >= thr_bits && smax != 0u)) {
+                        float sm_f = __builtin_bit_cast(float, smax);
+#pragma unroll
+                        for (int o = 32; o > 0; o >>= 1) sm_f = fmaxf(sm_f, __shfl_xor(sm_f, o, 64));
+                        const int e_tile = (int)((__builtin_bit_cast(uint32_t, sm_f) >> 23) & 0xFFu) - 126;
                         if (e_tile > e_run) {
                             if (e_run != E_NONE) ecorr = pow2i(e_run - e_tile);
                             e_run = e_tile;
+                            thr_bits = __builtin_bit_cast(uint32_t, pow2i(e_run));
+                            wfac = pow2i(WEXP - e_run);
                         }
                     }
                 }
-                const float wfac = e_run == E_NONE ? 0.0f : pow2i(WEXP - e_run);
                 u32x4 sw[2];                              // scale * 2^(WEXP - e_run) of the slots' keys, fp16 pairs
 #pragma unroll
                 for (int kh = 0; kh < 2; kh++) {
@@ -492,35 +578,38 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                     sw[kh][2] = pack_f16_rne(sv[kh][1][0] * wfac, sv[kh][1][1] * wfac);
                     sw[kh][3] = pack_f16_rne(sv[kh][1][2] * wfac, sv[kh][1][3] * wfac);
                 }
+                const uint32_t any_moved = (f0[0] | f0[1] | f0[2] | f0[3]) | (f1[0] | f1[1] | f1[2] | f1[3]);
+                if (__builtin_amdgcn_readfirstlane(any_moved) != 0u || ecorr != 1.0f) {
+                    // a scoring wave left the common reference in this tile (or the weights'
+                    // normaliser grew): bring accumulators and probabilities to the new maximum
 #pragma unroll
-                for (int h2 = 0; h2 < 2; h2++) {
-                    const float m_new = fmaxf(m_ref[h2], fmaxf(fmaxf(ml[h2][0], ml[h2][1]), fmaxf(ml[h2][2], ml[h2][3])));
-                    float fsel0 = 1.0f, fsel1 = 1.0f;
-                    const bool moved = __any(m_new != m_ref[h2] || ml[h2][0] != m_new || ml[h2][1] != m_new || ml[h2][2] != m_new || ml[h2][3] != m_new);
-                    if (moved || ecorr != 1.0f) {
+                    for (int h2 = 0; h2 < 2; h2++) {
+                        const f32x4 ml = LDS_AT(lds_f32x4, xb + xml_off + (uint32_t)(h2 * 256));
+                        const float m_new = fmaxf(m_ref[h2], fmaxf(fmaxf(ml[0], ml[1]), fmaxf(ml[2], ml[3])));
                         float f[4];
 #pragma unroll
-                        for (int k = 0; k < 4; k++) f[k] = ml[h2][k] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[h2][k] - m_new);
+                        for (int k = 0; k < 4; k++) f[k] = ml[k] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[k] - m_new);
                         const float c = (m_ref[h2] == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref[h2] - m_new)) * ecorr;
                         m_ref[h2] = m_new;
 #pragma unroll
                         for (int j = 0; j < 8; j++) oacc[h2][j] *= c;
                         // probabilities were taken relative to each key block's own reference: bring
                         // them to m_new (slot group g of half kh holds keys of key block 2 kh + g / 2)
-                        fsel0 = (g >> 1) ? f[1] : f[0];
-                        fsel1 = (g >> 1) ? f[3] : f[2];
-                    }
+                        const float fsel0 = (g >> 1) ? f[1] : f[0];
+                        const float fsel1 = (g >> 1) ? f[3] : f[2];
 #pragma unroll
-                    for (int kh = 0; kh < 2; kh++) {
-                        u32x4 swf = sw[kh];
-                        if (moved) {
+                        for (int kh = 0; kh < 2; kh++)
 #pragma unroll
-                            for (int d = 0; d < 4; d++) swf[d] = scale_f16x2(swf[d], kh ? fsel1 : fsel0);
-                        }
-#pragma unroll
-                        for (int d = 0; d < 4; d++) pw[h2][kh][d] = mul_f16x2(pw[h2][kh][d], swf[d]);
+                            for (int d = 0; d < 4; d++) pw[h2][kh][d] = scale_f16x2(pw[h2][kh][d], kh ? fsel1 : fsel0);
                     }
                 }
+#pragma unroll
+                for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+                    for (int kh = 0; kh < 2; kh++)
+#pragma unroll
+                        for (int d = 0; d < 4; d++) pw[h2][kh][d] = mul_f16x2(pw[h2][kh][d], sw[kh][d]);
+                const uint32_t va0 = tb + tr_off;
 #pragma unroll
                 for (int j0 = 0; j0 < 8; j0 += 4) {
                     i32x2 vt[4][2];
@@ -528,7 +617,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                     for (int j = 0; j < 4; j++)
 #pragma unroll
                         for (int kh = 0; kh < 2; kh++)
-                            vt[j][kh] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(vbase + (j0 + j) * (TK * 16) + kh * (32 * 16)));
+                            vt[j][kh] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(size_t)(va0 + (uint32_t)((j0 + j) * (TK * 16) + kh * (32 * 16))));
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -544,10 +633,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                         }
                 }
             }
-            // tile t+2 must be whole at the next barrier; the copies of tile t+3, issued in this
-            // step (eleven by value wave 0, ten by the others), may stay in flight
-            if (!do_copy) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NV) : "memory");
+            // tile t+2 must be whole at the next barrier; the share of tile t+3 issued in this
+            // step (four copies by waves 8, three by the others) may stay in flight.  Wave 11 has the
+            // whole of tile 2 in flight in step -1: it is needed one step later than tile 1.
+            if (do_copy) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+            else if (!(t < 0 && wave == 11)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             LDS_BARRIER();
         }
 
@@ -750,8 +840,11 @@ int run(Params &p, hipStream_t s, bool fixed = false) {
     static hipError_t attr_err = hipSuccess;
     const size_t smem = sizeof(Smem);
     std::call_once(attr_once, [&] {
-        attr_err = hipFuncSetAttribute((const void *)mla_roles_kernel,
+        attr_err = hipFuncSetAttribute((const void *)mla_roles_kernel<false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (attr_err == hipSuccess)
+            attr_err = hipFuncSetAttribute((const void *)mla_roles_kernel<true>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     });
     CWICK_HIP_CALL(attr_err);
     const int n_hb = (p.nh + HW - 1) / HW;
@@ -777,7 +870,8 @@ int run(Params &p, hipStream_t s, bool fixed = false) {
     }
     {
         ProfScope ps(fixed ? -1 : CWICK_HIP_PROF_MLA, s);
-        mla_roles_kernel<<<dim3((unsigned)total), THREADS, smem, s>>>(p);
+        if (p.sel) mla_roles_kernel<true><<<dim3((unsigned)total), THREADS, smem, s>>>(p);
+        else mla_roles_kernel<false><<<dim3((unsigned)total), THREADS, smem, s>>>(p);
     }
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
