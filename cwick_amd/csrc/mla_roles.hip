@@ -18,17 +18,32 @@
 //   The roles are one tile apart (tile t+1 is scored while tile t is accumulated), so a step has
 //   a single workgroup barrier and nobody waits for an exchange inside it.  The softmax
 //   reference is lazy: a scoring wave keeps the reference every wave knows (m_ref) unless its own
-//   tile exceeds it by 2^LAZY; the m it used travels with the probabilities, and the
-//   accumulating waves (and the scorers, for their sums) bring everything to the common maximum
-//   one step later -- almost always a comparison and nothing else.  Each scoring lane keeps the
-//   sum of its own keys; the sums meet once, after the loop.
-//   Tiles are copied global -> LDS by global_load_lds (no registers) into four stages: tile t+3
-//   is fetched during step t, two tiles ahead of its first use.  A wave that issues copies stalls
-//   while the memory pipeline takes them, so they go where there is slack: the value waves issue
-//   three each at the top of the step, the scoring waves the rest at the end of theirs, when they
-//   would otherwise wait at the barrier.  The copies are issued from inline assembly and the
-//   barrier waits for LDS traffic only, so the compiler never makes anything wait for the tiles
-//   in flight.
+//   tile exceeds it by 2^LAZY; the m it used travels with the probabilities together with one
+//   flag per scoring wave ("my reference for this tile is not the common one").  One step later
+//   every wave reads the eight flags: all clear (almost always) means nothing to do; otherwise
+//   the accumulating waves (and the scorers, for their sums) bring everything to the common
+//   maximum.  Each scoring lane keeps the sum of its own keys; the sums meet once, after the loop.
+//   Tiles are copied global -> LDS by global_load_lds (no registers) into four stages.  Tile 0 is
+//   fetched by all twelve waves at kernel start, tiles 1 and 2 by the two waves that have no part
+//   in the preparation of Q; from step 0 on every wave copies its share of tile t+3 during step t
+//   (three sixteen-byte columns of the 64 rows, plus a scale block for five of the waves): the
+//   value waves at the top of the step, the scoring waves at the end of theirs, when they would
+//   otherwise wait at the barrier.  The copies are issued from inline assembly and the barrier
+//   waits for LDS traffic only, so the compiler never makes anything wait for the tiles in
+//   flight.  LDS is addressed by integer byte offsets throughout (a generic pointer into LDS costs
+//   a null check and a 64-bit add per use), and the kernel exists in two instantiations: dense
+//   lists (rows are k_begin + i, only the last tile can be ragged) and lists given by sel[].
+//
+//   Where the time goes (counters and ablation builds, 12 waves on 256 CUs): a 64-key step takes
+//   about 3 000 cycles against 1 088 of matrix-core work.  Leaving out the tile copies, the score
+//   MFMAs or the value MFMAs with their conversions takes about a quarter off each, all three
+//   together two thirds; what remains (barrier, exchange, softmax, weights) is the last third.
+//   No single unit is saturated: vector ALU 56 % busy, matrix core 37 %, LDS 32 %.  The copy path
+//   of a compute unit moves a 38 KB tile in about 2 000 cycles when nothing else runs (18 bytes
+//   per cycle, the same from L2-resident rows, with contiguous instead of per-row accesses, and
+//   with loads staged through registers), so 32 query rows per tile cannot reach the matrix
+//   roof; 64 would halve the copies and the conversions per flop.  Eight or sixteen waves per
+//   workgroup (the same work split differently) were measured and are no faster.
 //
 //   LDS tile layout [16-byte column][key 0..63][16 B]: the K fragment is two 16-byte reads per
 //   lane, 256 B contiguous per 16 keys; the V^T fragment of 32 keys x 16 dims is one
@@ -252,10 +267,13 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     };
     auto share = [&](int r, uint32_t tile_off) {
         const uint64_t rp = row_ptr(r), sp = sc_ptr(r);
-        piece(wave, rp, sp, tile_off);
-        piece(wave + 12, rp, sp, tile_off);
-        piece(wave + 24, rp, sp, tile_off);
-        if (wave < NBLK) piece(NCOL + wave, rp, sp, tile_off);
+        // columns wave, wave + 12, wave + 24 (all below 36) and, for the first five waves, scale block `wave`
+        const uint32_t col_off = tile_off + (uint32_t)wave * (TK * 16);
+        const uint64_t col_src = rp + 16 * wave;
+        dma16(col_src, col_off);
+        dma16(col_src + 192, col_off + 12 * (TK * 16));
+        dma16(col_src + 384, col_off + 24 * (TK * 16));
+        if (wave < NBLK) dma4(sp + 4 * wave, tile_off + SC_OFF + (uint32_t)wave * (TK * 4));
         if (SEL && wave == 0) mark(r, tile_off);
     };
     auto whole = [&](int r, uint32_t tile_off) {
