@@ -117,6 +117,14 @@ int launch_quant_latent(const float *rows, int64_t n, uint8_t *out_rows, float *
 int launch_quant_ikeys(const float *rows, int64_t n, uint8_t *out_rows, float *out_scales,
                        hipStream_t s);
 int launch_narrow_bf16(const float *src, int64_t n, uint16_t *dst, hipStream_t s);
+int launch_mla_absorb(const uint16_t *kvb_w, const float *q, int64_t q_stride, int batch, int n_heads,
+                      int q_dim, int nope, int rope, int kv_dim, int kv_lora, uint16_t *q_abs, hipStream_t s);
+int launch_mla_expand(const uint16_t *kvb_w, const float *c_acc, int batch, int n_heads, int nope, int vdim,
+                      int kv_dim, int kv_lora, float *out, hipStream_t s);
+int launch_gqa_prepare(const float *q_proj, int64_t q_head_stride, const float *k_proj, const float *v_proj,
+                       int64_t n, int64_t pos0, int n_heads, int n_kv_heads, int head_dim, const float *q_norm,
+                       const float *k_norm, float eps, const float *rope_cos, const float *rope_sin, int rotary_dim,
+                       uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, hipStream_t s);
 int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
 int run_probe_hbm_read(size_t bytes, int reps, double *gbps);

@@ -983,6 +983,41 @@ const char *cwick_hip_prof_name(int which) {
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 
+int cwick_hip_mla_absorb_dev(const uint16_t *kv_b_proj, const float *q, int64_t q_batch_stride, int batch,
+                             int n_heads, int q_dim, int nope, int rope, int kv_dim, int kv_lora,
+                             uint16_t *q_abs, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_mla_absorb(kv_b_proj, q, q_batch_stride, batch, n_heads, q_dim, nope, rope, kv_dim, kv_lora,
+                             q_abs, (hipStream_t)stream);
+}
+
+int cwick_hip_mla_expand_dev(const uint16_t *kv_b_proj, const float *c_acc, int batch, int n_heads, int nope,
+                             int vdim, int kv_dim, int kv_lora, float *attn_out, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_mla_expand(kv_b_proj, c_acc, batch, n_heads, nope, vdim, kv_dim, kv_lora, attn_out,
+                             (hipStream_t)stream);
+}
+
+int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const float *k_proj,
+                              const float *v_proj, int64_t n, int64_t pos0, int n_heads, int n_kv_heads,
+                              int head_dim, const float *q_norm, const float *k_norm, float eps,
+                              const float *rope_cos, const float *rope_sin, int rotary_dim, uint16_t *q_out,
+                              cwick_hip_kv *cache, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    CWICK_REQUIRE(cache, "gqa_prepare: null cache");
+    CWICK_REQUIRE(n_kv_heads == cache->n_kv_heads && head_dim == cache->head_dim,
+                  "gqa_prepare: cache is %d x %d, call says %d x %d", cache->n_kv_heads, cache->head_dim, n_kv_heads,
+                  head_dim);
+    CWICK_REQUIRE(pos0 >= 0 && n >= 1 && pos0 + n <= cache->capacity, "gqa_prepare: rows %lld..%lld outside capacity %lld",
+                  (long long)pos0, (long long)(pos0 + n), (long long)cache->capacity);
+    return launch_gqa_prepare(q_proj, q_head_stride, k_proj, v_proj, n, pos0, n_heads, n_kv_heads, head_dim, q_norm,
+                              k_norm, eps, rope_cos, rope_sin, rotary_dim, q_out, cache->k, cache->v,
+                              (hipStream_t)stream);
+}
+
 int cwick_hip_probe_hbm_read(size_t bytes, int reps, double *gbps) {
     clear_error();
     if (!backend_ready()) return 0;   /* the reason is recorded */

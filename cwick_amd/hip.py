@@ -85,6 +85,10 @@ SIGNATURES = {
     "cwick_hip_dsa_decode_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _int, _i64,
                                         _vp, _vp, _int, _i64, _vp, _int, _flt, _vp, _vp, _vp,
                                         _vp]),
+    "cwick_hip_mla_absorb_dev": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _int, _vp, _vp]),
+    "cwick_hip_mla_expand_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _vp]),
+    "cwick_hip_gqa_prepare_dev": (_int, [_vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _flt,
+                                         _vp, _vp, _int, _vp, _vp, _vp]),
     "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
     "cwick_hip_probe_mfma": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
@@ -482,6 +486,26 @@ def dsa_decode_dev(ikeys, ikscale, key_bstride, kscale_bstride, rows, scales, ro
         row_bstride, scale_bstride, batch, n_keys, _dp(q_idx), _dp(w), n_idx_heads, topk_k,
         _dp(q), n_heads, scale, _dp(scores_tmp), _dp(sel_out), _dp(out), stream),
         "dsa_decode_dev")
+
+
+def mla_absorb_dev(kv_b_proj, q, q_bstride, batch, n_heads, q_dim, nope, rope, kv_dim, kv_lora, q_abs,
+                   stream=None):
+    return _check(lib().cwick_hip_mla_absorb_dev(_dp(kv_b_proj), _dp(q), q_bstride, batch, n_heads, q_dim,
+                                                 nope, rope, kv_dim, kv_lora, _dp(q_abs), stream),
+                  "mla_absorb_dev")
+
+
+def mla_expand_dev(kv_b_proj, c_acc, batch, n_heads, nope, vdim, kv_dim, kv_lora, out, stream=None):
+    return _check(lib().cwick_hip_mla_expand_dev(_dp(kv_b_proj), _dp(c_acc), batch, n_heads, nope, vdim,
+                                                 kv_dim, kv_lora, _dp(out), stream), "mla_expand_dev")
+
+
+def gqa_prepare_dev(q_proj, q_head_stride, k_proj, v_proj, n, pos0, n_heads, n_kv_heads, head_dim,
+                    q_norm, k_norm, eps, rope_cos, rope_sin, rotary_dim, q_out, cache, stream=None, raw=False):
+    rc = lib().cwick_hip_gqa_prepare_dev(_dp(q_proj), q_head_stride, _dp(k_proj), _dp(v_proj), n, pos0,
+                                         n_heads, n_kv_heads, head_dim, _dp(q_norm), _dp(k_norm), eps,
+                                         _dp(rope_cos), _dp(rope_sin), rotary_dim, _dp(q_out), cache.h, stream)
+    return rc if raw else _check(rc, "gqa_prepare_dev")
 
 
 # ------------------------------------------------------------------ phase timers

@@ -324,6 +324,49 @@ int cwick_hip_dsa_decode_dev(const uint8_t *ikeys, const float *ikscale,
                              float scale, float *scores_tmp, int32_t *sel_out, float *out,
                              void *stream);
 
+/* ---- the steps around the attention kernels, on HBM-resident operands ---- */
+/* With these the queries and the attention outputs never cross the host link:
+ * the projections' outputs go in, what the attention kernels take comes out. */
+
+/* Replaces the absorb loop of mla_latent_decode (src/attention.c:741-744,
+ * gemv_bf16_t :145-177): q_abs[h][c] = sum_i q[h][i] * W_k[h][i][c] for the
+ * `nope` leading dims of every head's query, W_k[h] = rows h*kv_dim ..
+ * h*kv_dim+nope of kv_b_proj (bf16, row-major [n_heads*kv_dim][kv_lora]);
+ * the `rope` dims that follow in q pass through to q_abs[h][512 .. 512+rope)
+ * (zero-filled to 576).  q fp32 [batch][n_heads][q_dim] (batch stride in
+ * floats), q_abs bf16 [batch][n_heads][576], rounded to nearest even: the
+ * query operand of cwick_hip_mla_decode_dev.  kv_lora must be 512. */
+int cwick_hip_mla_absorb_dev(const uint16_t *kv_b_proj, const float *q, int64_t q_batch_stride,
+                             int batch, int n_heads, int q_dim, int nope, int rope, int kv_dim,
+                             int kv_lora, uint16_t *q_abs, void *stream);
+
+/* Replaces the expansion after the accumulation (src/attention.c:812-815,
+ * gemv_bf16_n :184-224): attn_out[h][r] = W_v[h][r] . c_acc[h], W_v[h] = rows
+ * h*kv_dim+nope .. +vdim of kv_b_proj.  c_acc fp32 [batch][n_heads][512] (the
+ * output of the MLA kernels), attn_out fp32 [batch][n_heads][vdim]. */
+int cwick_hip_mla_expand_dev(const uint16_t *kv_b_proj, const float *c_acc, int batch, int n_heads,
+                             int nope, int vdim, int kv_dim, int kv_lora, float *attn_out,
+                             void *stream);
+
+/* Replaces the per-token loop of mixer_attn between the projections and the
+ * attention (src/q35_model.c:1627-1652): for each of n tokens at positions
+ * pos0.., every query head and every key head is RMS-normalised with (1 + w)
+ * weights (rms_norm_w, :111-121; a NULL weight means no weight) and its first
+ * rotary_dim dims are rotated, rotate-half form (rope_apply, :144-153), with
+ * the cos/sin tables of build_rope (:459-476), [position][rotary_dim/2] fp32.
+ * q_proj fp32 [n][n_heads] heads q_head_stride floats apart (2*head_dim when
+ * the projection carries a gate per head, :1634-1637), k_proj and v_proj fp32
+ * [n][n_kv_heads*head_dim].  q_out bf16 [n][n_heads][head_dim] is the query
+ * operand of cwick_hip_gqa_decode_dev / _prefill_dev; the K and V rows are
+ * narrowed to bf16 and stored into rows pos0.. of `cache` (the memcpy pair of
+ * :1649-1651).  head_dim <= 256. */
+int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const float *k_proj,
+                              const float *v_proj, int64_t n, int64_t pos0, int n_heads,
+                              int n_kv_heads, int head_dim, const float *q_norm,
+                              const float *k_norm, float eps, const float *rope_cos,
+                              const float *rope_sin, int rotary_dim, uint16_t *q_out,
+                              cwick_hip_kv *cache, void *stream);
+
 /* ---- phase timers ------------------------------------------------------- */
 /* Replace the reference's attention sub-timers (g_attn_*_ns, src/attention.c:1169-1174,
  * read out by src/prof.c:184-196 under CWICK_PROFILE; CWICK_Q35_PROF's

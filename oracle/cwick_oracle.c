@@ -48,6 +48,13 @@
  *                                      PARITY UNPINNED against a reference build
  *   orc_mla_prefill_chunk              loop-of-decodes identity, bit for bit: PARITY
  *                                      UNPINNED against a reference build
+ *   orc_mla_absorb, orc_mla_expand     double brute force (a transposed or mis-sliced weight
+ *                                      fails), the absorption identity: scores from q_abs over
+ *                                      the latent equal scores from q over W_k-expanded keys
+ *   orc_gqa_prepare, orc_build_rope    closed forms (norm of a constant head, rotation by a
+ *                                      quarter turn, position 0 is the identity), double
+ *                                      brute force, norm preserved by the rotation:
+ *                                      PARITY UNPINNED against a reference build
  *   orc_indexer_scores[_ds]            double brute force, ReLU-before-weight, thread
  *                                      count invariance: PARITY UNPINNED against a
  *                                      reference build
@@ -743,6 +750,116 @@ ORC_API void orc_sparse_attn_sink(const uint16_t *q_bf16,   /* [nh][kdim] */
         free(sc); free(qh);
     }
     free(rows);
+}
+
+/* ------------------------------------------------------------------ */
+/* the steps around the attention kernels                               */
+/* ------------------------------------------------------------------ */
+/* src/attention.c:145-177 (gemv_bf16_t, the portable loop at :170-176) applied per head as at
+ * :741-744: q_abs[h][c] = sum_r q[h][r] * W_k[h][r][c], row-outer, rows whose q is zero
+ * skipped, multiply and add rounded separately.  W_k[h] = rows h*kv_dim .. +nope of kv_b_proj.
+ * The `rope` dims that follow the nope dims in q are copied behind the kv_lora outputs (the
+ * reference's released model has none, :107); the row is padded to `out_dim` with zeros. */
+ORC_API void orc_mla_absorb(const uint16_t *kvb_w, const float *q, int nh, int q_dim, int nope,
+                            int rope, int kv_dim, int kv_lora, int out_dim, float *q_abs) {
+    for (int h = 0; h < nh; h++) {
+        float *out = q_abs + (size_t)h * out_dim;
+        const float *in = q + (size_t)h * q_dim;
+        const uint16_t *w = kvb_w + (size_t)h * kv_dim * kv_lora;
+        for (int c = 0; c < out_dim; c++) out[c] = 0.0f;
+        for (int r = 0; r < nope; r++) {
+            const float a = in[r];
+            if (a == 0.0f) continue;
+            const uint16_t *wr = w + (size_t)r * kv_lora;
+            for (int c = 0; c < kv_lora; c++) out[c] += a * orc_bf16_to_f32(wr[c]);
+        }
+        for (int i = 0; i < rope && kv_lora + i < out_dim; i++) out[kv_lora + i] = in[nope + i];
+    }
+}
+
+/* src/attention.c:184-224 (gemv_bf16_n, the portable loop at :211-223: four partial sums over
+ * j mod 4, combined (s0+s1)+(s2+s3)) applied per head as at :812-815:
+ * attn_out[h][r] = W_v[h][r] . c_acc[h], W_v[h] = rows h*kv_dim+nope .. +vdim of kv_b_proj. */
+ORC_API void orc_mla_expand(const uint16_t *kvb_w, const float *c_acc, int nh, int nope, int vdim,
+                            int kv_dim, int kv_lora, float *attn_out) {
+    for (int h = 0; h < nh; h++) {
+        const float *in = c_acc + (size_t)h * kv_lora;
+        for (int r = 0; r < vdim; r++) {
+            const uint16_t *wr = kvb_w + ((size_t)h * kv_dim + nope + r) * kv_lora;
+            float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+            int j = 0;
+            for (; j + 4 <= kv_lora; j += 4) {
+                s0 += orc_bf16_to_f32(wr[j + 0]) * in[j + 0];
+                s1 += orc_bf16_to_f32(wr[j + 1]) * in[j + 1];
+                s2 += orc_bf16_to_f32(wr[j + 2]) * in[j + 2];
+                s3 += orc_bf16_to_f32(wr[j + 3]) * in[j + 3];
+            }
+            for (; j < kv_lora; j++) s0 += orc_bf16_to_f32(wr[j]) * in[j];
+            attn_out[(size_t)h * vdim + r] = (s0 + s1) + (s2 + s3);
+        }
+    }
+}
+
+/* src/q35_model.c:459-476 (build_rope): cos/sin of p / theta^(2i/rotary) in double, stored as
+ * float, [position][rotary/2]. */
+ORC_API void orc_build_rope(int max_pos, int rotary, double theta, float *cos_t, float *sin_t) {
+    const int pairs = rotary / 2;
+    for (int p = 0; p < max_pos; p++)
+        for (int i = 0; i < pairs; i++) {
+            const double inv = 1.0 / pow(theta, (double)(2 * i) / (double)rotary);
+            const double a = (double)p * inv;
+            cos_t[(size_t)p * pairs + i] = (float)cos(a);
+            sin_t[(size_t)p * pairs + i] = (float)sin(a);
+        }
+}
+
+/* src/q35_model.c:111-121 (rms_norm_w: serial sum of squares, rstd = 1/sqrtf(acc/n + eps),
+ * out = in * rstd * (1 + w)) followed by :144-153 (rope_apply: index i pairs with i + pairs,
+ * rotate-half) on one head, in place; w may be NULL. */
+static void orc_head_norm_rope(float *v, int hd, const float *w, float eps, const float *cos_p,
+                               const float *sin_p, int rotary) {
+    float acc = 0.0f;
+    for (int i = 0; i < hd; i++) acc += v[i] * v[i];
+    const float rstd = 1.0f / sqrtf(acc / (float)hd + eps);
+    if (w) for (int i = 0; i < hd; i++) v[i] = v[i] * rstd * (1.0f + w[i]);
+    else for (int i = 0; i < hd; i++) v[i] = v[i] * rstd;
+    const int pairs = rotary / 2;
+    for (int i = 0; i < pairs; i++) {
+        const float c = cos_p[i], s = sin_p[i];
+        const float a = v[i], b = v[i + pairs];
+        v[i] = a * c - b * s;
+        v[i + pairs] = b * c + a * s;
+    }
+}
+
+/* src/q35_model.c:1627-1652: the per-token loop of mixer_attn between the projections and the
+ * attention.  q_proj heads are q_head_stride floats apart (the gate sits behind each head's
+ * query when there is one).  Outputs are narrowed to bf16 with round-to-nearest-even (what the
+ * device caches and kernels hold): q_out [n][H][HD], k_rows / v_rows [n][KV*HD]. */
+ORC_API void orc_gqa_prepare(const float *q_proj, int64_t q_head_stride, const float *k_proj,
+                             const float *v_proj, int64_t n, int64_t pos0, int H, int KV, int HD,
+                             const float *q_norm, const float *k_norm, float eps,
+                             const float *rope_cos, const float *rope_sin, int rotary,
+                             uint16_t *q_out, uint16_t *k_rows, uint16_t *v_rows) {
+    const int pairs = rotary / 2;
+    float *tmp = malloc(sizeof(float) * (size_t)HD);
+    for (int64_t t = 0; t < n; t++) {
+        const float *cos_p = rope_cos + (size_t)(pos0 + t) * pairs;
+        const float *sin_p = rope_sin + (size_t)(pos0 + t) * pairs;
+        for (int h = 0; h < H; h++) {
+            memcpy(tmp, q_proj + ((size_t)t * H + h) * q_head_stride, sizeof(float) * (size_t)HD);
+            orc_head_norm_rope(tmp, HD, q_norm, eps, cos_p, sin_p, rotary);
+            for (int i = 0; i < HD; i++) q_out[((size_t)t * H + h) * HD + i] = orc_f32_to_bf16_rne(tmp[i]);
+        }
+        for (int h = 0; h < KV; h++) {
+            memcpy(tmp, k_proj + ((size_t)t * KV + h) * HD, sizeof(float) * (size_t)HD);
+            orc_head_norm_rope(tmp, HD, k_norm, eps, cos_p, sin_p, rotary);
+            for (int i = 0; i < HD; i++) k_rows[((size_t)t * KV + h) * HD + i] = orc_f32_to_bf16_rne(tmp[i]);
+        }
+        for (int i = 0; i < KV * HD; i++)
+            v_rows[(size_t)t * KV * HD + i] = orc_f32_to_bf16_rne(v_proj[(size_t)t * KV * HD + i]);
+    }
+    free(tmp);
 }
 
 /* ------------------------------------------------------------------ */

@@ -260,6 +260,52 @@ def sparse_attn_sink(q, lat, scales, scale, sink=None, sel=None, nlist=None, nth
     return out
 
 
+def mla_absorb(kvb_w, q, nope, rope, kv_dim, kv_lora=512, out_dim=KDIM):
+    """q [nh, q_dim] f32, kvb_w [nh*kv_dim, kv_lora] u16 -> q_abs [nh, out_dim] f32."""
+    kvb_w = np.ascontiguousarray(kvb_w, np.uint16)
+    q = np.ascontiguousarray(q, np.float32)
+    nh, q_dim = q.shape
+    out = np.empty((nh, out_dim), np.float32)
+    lib().orc_mla_absorb(_p(kvb_w, C.c_uint16), _p(q, C.c_float), nh, q_dim, nope, rope, kv_dim, kv_lora,
+                         out_dim, _p(out, C.c_float))
+    return out
+
+
+def mla_expand(kvb_w, c_acc, nope, vdim, kv_dim, kv_lora=512):
+    kvb_w = np.ascontiguousarray(kvb_w, np.uint16)
+    c_acc = np.ascontiguousarray(c_acc, np.float32)
+    nh = c_acc.shape[0]
+    out = np.empty((nh, vdim), np.float32)
+    lib().orc_mla_expand(_p(kvb_w, C.c_uint16), _p(c_acc, C.c_float), nh, nope, vdim, kv_dim, kv_lora,
+                         _p(out, C.c_float))
+    return out
+
+
+def build_rope(max_pos, rotary, theta):
+    cos_t = np.empty((max_pos, rotary // 2), np.float32)
+    sin_t = np.empty((max_pos, rotary // 2), np.float32)
+    lib().orc_build_rope(max_pos, rotary, C.c_double(theta), _p(cos_t, C.c_float), _p(sin_t, C.c_float))
+    return cos_t, sin_t
+
+
+def gqa_prepare(q_proj, q_head_stride, k_proj, v_proj, pos0, H, KV, HD, q_norm, k_norm, eps, cos_t, sin_t, rotary):
+    q_proj = np.ascontiguousarray(q_proj, np.float32)
+    k_proj = np.ascontiguousarray(k_proj, np.float32)
+    v_proj = np.ascontiguousarray(v_proj, np.float32)
+    n = k_proj.shape[0]
+    qo = np.empty((n, H, HD), np.uint16)
+    ko = np.empty((n, KV * HD), np.uint16)
+    vo = np.empty((n, KV * HD), np.uint16)
+    qn = None if q_norm is None else _p(np.ascontiguousarray(q_norm, np.float32), C.c_float)
+    kn = None if k_norm is None else _p(np.ascontiguousarray(k_norm, np.float32), C.c_float)
+    lib().orc_gqa_prepare(_p(q_proj, C.c_float), C.c_int64(q_head_stride), _p(k_proj, C.c_float),
+                          _p(v_proj, C.c_float), C.c_int64(n), C.c_int64(pos0), H, KV, HD, qn, kn,
+                          C.c_float(eps), _p(np.ascontiguousarray(cos_t, np.float32), C.c_float),
+                          _p(np.ascontiguousarray(sin_t, np.float32), C.c_float), rotary,
+                          _p(qo, C.c_uint16), _p(ko, C.c_uint16), _p(vo, C.c_uint16))
+    return qo, ko, vo
+
+
 def topk_contract(sc, k):
     sc = np.ascontiguousarray(sc, np.float32)
     out = np.empty(max(min(k, sc.size), 1), np.int32)

@@ -736,3 +736,108 @@ def test_indexer_scores_ds_mode_bit_exact(hip, orc, n_keys, ih):
     rc, _ = hip.indexer_scores(cache, 0, n_keys, q, w, mode=7, raw=True)
     assert rc == 0 and "mode" in hip.last_error()
     cache.free()
+
+
+# ------------------------------------------------------------------ the steps around the attention kernels
+def test_mla_absorb_decode_expand_chain_on_device(hip, orc):
+    """W_k absorb -> MLA decode -> W_v expand with every intermediate in HBM (the absorbed query
+    and c_acc never cross the host link): src/attention.c:741-744, :749-811, :812-815.  Each
+    device step is compared with the oracle's restatement on its own (absorb and expand to fp32
+    rounding: the GPU sums in a different order; tolerance 1e-4 relative to the largest value,
+    plus the bf16 rounding of q_abs), and the chain as a whole with the oracle's chain."""
+    import torch
+    say("[case] absorb -> decode -> expand on the device")
+    nh, nope, rope, vdim, kv_lora, n_keys = 128, 128, 64, 128, 512, 3000
+    q_dim, kv_dim = nope + rope, nope + vdim
+    g = synth.rng(1234)
+    kvb = synth.f32_to_bf16(g.standard_normal((nh * kv_dim, kv_lora), dtype=np.float32) * np.float32(kv_lora ** -0.5))
+    q = g.standard_normal((nh, q_dim), dtype=np.float32)
+    c = synth.cfg3_mla_decode(n_keys, nh, seed=1235)
+    s = torch.cuda.current_stream().cuda_stream
+    d_kvb = torch.from_numpy(kvb.view(np.int16)).cuda()
+    d_q = torch.from_numpy(q).cuda()
+    d_qabs = torch.empty((nh, synth.KDIM), dtype=torch.int16, device="cuda")
+    d_rows = torch.from_numpy(c["rows"]).cuda(); d_scales = torch.from_numpy(c["scales"]).cuda()
+    d_cacc = torch.empty((nh, synth.VDIM), dtype=torch.float32, device="cuda")
+    d_out = torch.empty((nh, vdim), dtype=torch.float32, device="cuda")
+    hip.mla_absorb_dev(d_kvb, d_q, 0, 1, nh, q_dim, nope, rope, kv_dim, kv_lora, d_qabs, s)
+    hip.mla_decode_dev(d_rows, d_scales, 0, 0, n_keys, 1, None, n_keys, d_qabs, nh, c["scale"], d_cacc, s)
+    hip.mla_expand_dev(d_kvb, d_cacc, 1, nh, nope, vdim, kv_dim, kv_lora, d_out, s)
+    torch.cuda.synchronize()
+    # absorb
+    qabs_ref = orc.mla_absorb(kvb, q, nope, rope, kv_dim)
+    qabs_got = synth.bf16_to_f32(d_qabs.cpu().numpy().view(np.uint16))
+    scale_q = np.abs(qabs_ref).max()
+    assert np.abs(qabs_got - qabs_ref).max() <= 2.0 ** -8 * scale_q + 1e-4 * scale_q        # bf16 rounding of the output
+    assert np.array_equal(qabs_got[:, 512:], synth.bf16_to_f32(synth.f32_to_bf16(q[:, nope:])))
+    # decode from the device's own q_abs bits
+    qabs_bits = d_qabs.cpu().numpy().view(np.uint16)
+    cacc_ref = orc.mla_decode(qabs_bits, c["rows"], c["scales"], c["scale"], nthreads=0)
+    cacc_got = d_cacc.cpu().numpy()
+    assert_close(cacc_got, cacc_ref, "decode inside the device chain")
+    # expand from the device's own c_acc
+    out_ref = orc.mla_expand(kvb, cacc_got, nope, vdim, kv_dim)
+    out_got = d_out.cpu().numpy()
+    assert np.abs(out_got - out_ref).max() <= 1e-4 * np.abs(out_ref).max()
+    # the chain against the oracle's chain (q_abs narrowed to bf16 there as well)
+    chain = orc.mla_expand(kvb, orc.mla_decode(synth.f32_to_bf16(qabs_ref), c["rows"], c["scales"], c["scale"],
+                                               nthreads=0), nope, vdim, kv_dim)
+    assert_close(out_got, chain, "absorb -> decode -> expand")
+    # a latent width other than 512 is declined
+    rc = hip.lib().cwick_hip_mla_absorb_dev(d_kvb.data_ptr(), d_q.data_ptr(), 0, 1, nh, q_dim, nope, rope, kv_dim,
+                                            256, d_qabs.data_ptr(), s)
+    assert rc == 0 and "kv_lora" in hip.last_error()
+
+
+@pytest.mark.parametrize("n,pos0,H,KV,HD,rotary,gate", [(1, 4095, 16, 4, 256, 64, True), (300, 100, 16, 4, 256, 64, True),
+                                                       (17, 0, 8, 8, 128, 128, False), (5, 9, 4, 2, 256, 0, False)])
+def test_gqa_prepare_on_device_then_attention(hip, orc, n, pos0, H, KV, HD, rotary, gate):
+    """q/k head norm + RoPE + narrowing + cache append on the device (src/q35_model.c:1627-1652),
+    then attention over the rows it appended, queries never leaving HBM.  The prepared values
+    agree with the oracle's to one bf16 step (the sum of squares is a wave's tree sum here and a
+    serial loop there: tolerance 2^-7 relative per head, stated)."""
+    import torch
+    say("[case] gqa_prepare", n, pos0, H, KV, HD, rotary, gate)
+    g = synth.rng(4321 + n)
+    stride = HD * (2 if gate else 1)
+    theta, eps = 1e6, 1e-6
+    cos_t, sin_t = orc.build_rope(pos0 + n, max(rotary, 2), theta)
+    qp = g.standard_normal((n, H, stride), dtype=np.float32)
+    kp = g.standard_normal((n, KV * HD), dtype=np.float32)
+    vp = g.standard_normal((n, KV * HD), dtype=np.float32)
+    qn = (g.standard_normal(HD, dtype=np.float32) * np.float32(0.1))
+    kn = (g.standard_normal(HD, dtype=np.float32) * np.float32(0.1))
+    cache = hip.KVCache(pos0 + n, KV, HD)
+    if pos0:
+        past = synth.cfg2_gqa_prefill(pos0, H, KV, HD, 0, seed=99)
+        cache.write(0, past["k"].reshape(pos0, -1), past["v"].reshape(pos0, -1))
+    s = torch.cuda.current_stream().cuda_stream
+    d = lambda a: torch.from_numpy(a).cuda()
+    d_q = torch.empty((n, H, HD), dtype=torch.int16, device="cuda")
+    hip.gqa_prepare_dev(d(qp), stride, d(kp), d(vp), n, pos0, H, KV, HD, d(qn), d(kn), eps, d(cos_t), d(sin_t),
+                        rotary, d_q, cache, s)
+    torch.cuda.synchronize()
+    q_got = d_q.cpu().numpy().view(np.uint16)
+    k_got, v_got = cache.read(pos0, n)
+    q_ref, k_ref, v_ref = orc.gqa_prepare(qp, stride, kp, vp, pos0, H, KV, HD, qn, kn, eps, cos_t, sin_t, rotary)
+    assert np.array_equal(v_got, v_ref)                           # narrowing only: bit for bit
+    for got, ref, heads in ((q_got.reshape(n, H, HD), q_ref.reshape(n, H, HD), H),
+                            (k_got.reshape(n, KV, HD), k_ref.reshape(n, KV, HD), KV)):
+        gf, rf = synth.bf16_to_f32(got), synth.bf16_to_f32(ref)
+        tol = 2.0 ** -7 * np.abs(rf).max(axis=-1, keepdims=True)
+        assert (np.abs(gf - rf) <= tol).all(), "prepared heads differ by more than a bf16 step"
+        assert (got != ref).mean() < 0.02, "more than 2 %% of the prepared values differ from the oracle's bits"
+    if HD == 256 and KV * 4 >= H:
+        # attention straight from the prepared queries and the appended rows
+        out = torch.empty((n, H, HD), dtype=torch.float32, device="cuda")
+        scale = float(HD) ** -0.5
+        hip.gqa_prefill_dev(cache.k_dev(), cache.v_dev(), pos0, n, KV, HD, d_q, H, scale, out, s)
+        torch.cuda.synchronize()
+        k_all, v_all = cache.read(0, pos0 + n)
+        ref = orc.gqa_prefill(q_got.reshape(n, H, HD), k_all.reshape(-1, KV, HD), v_all.reshape(-1, KV, HD), pos0, scale,
+                              nthreads=0)
+        assert_close(out.cpu().numpy(), ref, "gqa_prefill over prepared queries and rows")
+    rc = hip.gqa_prepare_dev(d(qp), stride, d(kp), d(vp), n, pos0 + 1, H, KV, HD, d(qn), d(kn), eps, d(cos_t), d(sin_t),
+                             rotary, d_q, cache, s, raw=True)
+    assert rc == 0 and "capacity" in hip.last_error()
+    cache.free()

@@ -282,3 +282,82 @@ def test_indexer_scores_ds_vs_brute_force(orc):
     assert np.abs(got - want).max() > 1e-5            # ... and is really there
     # threads only split the keys
     assert np.array_equal(got, orc.indexer_scores_ds(q, w, keys, ks, nthreads=0))
+
+
+# ------------------------------------------------------------------ the steps around the kernels
+def test_mla_absorb_expand_vs_brute_force(orc):
+    """gemv_bf16_t / gemv_bf16_n per head (src/attention.c:741-744, :812-815).  Brute force in
+    double with the weight slices taken independently; the absorption identity the reference
+    itself checks (:838-893): scores of q_abs against the latent equal scores of q against the
+    keys expanded through W_k."""
+    g = synth.rng(51)
+    nh, nope, rope, vdim, kv_lora = 6, 40, 8, 24, 512
+    q_dim, kv_dim = nope + rope, nope + vdim
+    kvb = synth.normal_bf16(g, (nh * kv_dim, kv_lora))
+    q = g.standard_normal((nh, q_dim)).astype(np.float32)
+    q[2, 5] = 0.0                                            # a skipped row
+    W = f32(kvb).reshape(nh, kv_dim, kv_lora)
+    got = orc.mla_absorb(kvb, q, nope, rope, kv_dim)
+    want = np.einsum("hr,hrc->hc", q[:, :nope].astype(np.float64), W[:, :nope])
+    assert got.shape == (nh, 576)
+    assert np.abs(got[:, :512] - want).max() < 1e-4
+    assert np.array_equal(got[:, 512:512 + rope], q[:, nope:]) and not got[:, 512 + rope:].any()
+    # transposed or mis-sliced weights would give something else entirely
+    assert np.abs(want - np.einsum("hr,hrc->hc", q[:, :nope].astype(np.float64), W[:, vdim:vdim + nope])).max() > 1.0
+    c = g.standard_normal((nh, kv_lora)).astype(np.float32)
+    ex = orc.mla_expand(kvb, c, nope, vdim, kv_dim)
+    assert np.abs(ex - np.einsum("hrc,hc->hr", W[:, nope:], c.astype(np.float64))).max() < 1e-4
+    # absorption identity: (W_k^T q) . c == q . (W_k c)
+    lat = g.standard_normal((9, kv_lora))
+    s_abs = got[:, :512].astype(np.float64) @ lat.T
+    s_exp = np.einsum("hr,thr->ht", q[:, :nope].astype(np.float64), np.einsum("hrc,tc->thr", W[:, :nope], lat))
+    assert np.abs(s_abs - s_exp).max() < 1e-3
+
+
+def test_gqa_prepare_closed_forms_and_brute_force(orc):
+    """rms_norm_w with (1 + w) weights, rotate-half RoPE on the first rotary dims, bf16 narrowing
+    (src/q35_model.c:1627-1652)."""
+    H, KV, HD, rotary, theta, eps = 4, 2, 64, 32, 10000.0, 1e-6
+    cos_t, sin_t = orc.build_rope(50, rotary, theta)
+    inv = 1.0 / theta ** (2 * np.arange(rotary // 2) / rotary)
+    assert np.allclose(cos_t[7], np.cos(7 * inv), atol=1e-7) and np.allclose(sin_t[7], np.sin(7 * inv), atol=1e-7)
+    assert (cos_t[0] == 1).all() and (sin_t[0] == 0).all()
+    g = synth.rng(52)
+    n, pos0 = 5, 3
+    stride = 2 * HD                                            # a gate behind every head's query
+    qp = g.standard_normal((n, H, stride)).astype(np.float32)
+    kp = g.standard_normal((n, KV * HD)).astype(np.float32)
+    vp = g.standard_normal((n, KV * HD)).astype(np.float32)
+    qn = (g.standard_normal(HD) * 0.1).astype(np.float32)
+    kn = (g.standard_normal(HD) * 0.1).astype(np.float32)
+    qo, ko, vo = orc.gqa_prepare(qp, stride, kp, vp, pos0, H, KV, HD, qn, kn, eps, cos_t, sin_t, rotary)
+
+    def brute(x, w, p):
+        x = x.astype(np.float64)
+        y = x / np.sqrt((x * x).mean() + eps) * (1.0 + w.astype(np.float64))
+        half = rotary // 2
+        a, b = y[:half].copy(), y[half:rotary].copy()
+        c, s_ = np.cos(p * inv), np.sin(p * inv)
+        y[:half], y[half:rotary] = a * c - b * s_, b * c + a * s_
+        return y
+    for t in range(n):
+        for h in range(H):
+            want = brute(qp[t, h, :HD], qn, pos0 + t)
+            assert np.abs(synth.bf16_to_f32(qo[t, h]) - want).max() < 2.0 ** -7 * np.abs(want).max()
+        for h in range(KV):
+            want = brute(kp[t, h * HD:(h + 1) * HD], kn, pos0 + t)
+            assert np.abs(synth.bf16_to_f32(ko[t, h * HD:(h + 1) * HD]) - want).max() < 2.0 ** -7 * np.abs(want).max()
+    assert np.array_equal(vo, synth.f32_to_bf16(vp))
+    # closed forms: a constant head normalises to +-1 (times 1 + w); the gate half is never read
+    one = np.full((1, 1, stride), 3.0, np.float32)
+    one[0, 0, HD:] = 1e9
+    z = np.zeros((1, HD), np.float32)
+    q1, _, _ = orc.gqa_prepare(one, stride, z, z, 0, 1, 1, HD, None, None, 0.0, cos_t, sin_t, rotary)
+    assert np.array_equal(synth.bf16_to_f32(q1[0, 0]), np.ones(HD, np.float32))
+    # a quarter turn: with cos = 0, sin = 1 the two halves swap with a sign
+    c0 = np.zeros((1, rotary // 2), np.float32); s1 = np.ones((1, rotary // 2), np.float32)
+    x = np.zeros((1, 1, HD), np.float32); x[0, 0, :HD] = np.arange(1, HD + 1)
+    q2, _, _ = orc.gqa_prepare(x, HD, z, z, 0, 1, 1, HD, None, None, 0.0, c0, s1, rotary)
+    y = x[0, 0] / np.sqrt((x[0, 0] ** 2).mean())
+    want = y.copy(); want[:rotary // 2] = -y[rotary // 2:rotary]; want[rotary // 2:rotary] = y[:rotary // 2]
+    assert np.abs(synth.bf16_to_f32(q2[0, 0]) - want).max() < 2.0 ** -7 * np.abs(want).max()
