@@ -125,6 +125,14 @@ int launch_gqa_prepare(const float *q_proj, int64_t q_head_stride, const float *
                        int64_t n, int64_t pos0, int n_heads, int n_kv_heads, int head_dim, const float *q_norm,
                        const float *k_norm, float eps, const float *rope_cos, const float *rope_sin, int rotary_dim,
                        uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, hipStream_t s);
+int launch_ikeys_pool(const float *tail_k, const float *tail_g, const uint16_t *ape, const float *knw, const float *knb,
+                      float eps, int kpool, int64_t n_pools, uint8_t *out_rows, float *out_scales, float *out_f32,
+                      hipStream_t s);
+int launch_candidate_select(const float *scores, int batch, int64_t n, int block, int64_t topk_blocks, uint8_t *cand,
+                            hipStream_t s);
+int launch_candidate_apply(float *scores, const uint8_t *cand, int batch, int64_t n, hipStream_t s);
+int launch_dequant_latent(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
+int launch_dequant_ikeys(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
 int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
 int run_probe_hbm_read(size_t bytes, int reps, double *gbps);
@@ -206,6 +214,40 @@ __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Round-to-nearest-even fp32 -> E4M3fn (the caller has clamped to +-448): the
+// bit recipe of src/ds_quant.c:102-128, except that a round-up out of the last
+// subnormal carries into the first normal (byte 0x08) instead of being masked
+// away (`mm & 7u`, :127), so that the result is the nearest grid point as the
+// reference's own round-trip check demands (tools/ds_verify.c:48-63).
+__device__ __forceinline__ uint32_t f32_to_e4m3_rne(float v) {
+    if (v == 0.0f) return 0u;
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    uint32_t sign = u >> 31;
+    int32_t exp = (int32_t)((u >> 23) & 0xFFu) - 127;
+    uint32_t m24 = (1u << 23) | (u & 0x7FFFFFu);
+    if (exp >= -6) {
+        uint32_t keep = m24 >> 20;
+        uint32_t rem = m24 & 0xFFFFFu;
+        if (rem > 0x80000u || (rem == 0x80000u && (keep & 1u))) keep++;
+        int32_t e = exp;
+        if (keep == 16u) { keep >>= 1; e++; }
+        if (e > 8) { keep = 14u; e = 8; }
+        return (sign << 7) | ((uint32_t)(e + 7) << 3) | (keep & 7u);
+    }
+    if (exp < -10) return sign << 7;
+    int32_t sh = 14 - exp;
+    uint32_t mm = m24 >> sh;
+    uint32_t rem = m24 & ((1u << sh) - 1u);
+    uint32_t half = 1u << (sh - 1);
+    if (rem > half || (rem == half && (mm & 1u))) mm++;
+    return (sign << 7) | mm;
 }
 
 }  // namespace cwick

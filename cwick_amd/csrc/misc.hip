@@ -5,35 +5,6 @@
 
 namespace cwick {
 
-// Round-to-nearest-even fp32 -> E4M3fn (the caller has clamped to +-448): the
-// bit recipe of src/ds_quant.c:102-128, except that a round-up out of the last
-// subnormal carries into the first normal (byte 0x08) instead of being masked
-// away (`mm & 7u`, :127), so that the result is the nearest grid point as the
-// reference's own round-trip check demands (tools/ds_verify.c:48-63).
-__device__ __forceinline__ uint32_t f32_to_e4m3_rne(float v) {
-    if (v == 0.0f) return 0u;
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    uint32_t sign = u >> 31;
-    int32_t exp = (int32_t)((u >> 23) & 0xFFu) - 127;
-    uint32_t m24 = (1u << 23) | (u & 0x7FFFFFu);
-    if (exp >= -6) {
-        uint32_t keep = m24 >> 20;
-        uint32_t rem = m24 & 0xFFFFFu;
-        if (rem > 0x80000u || (rem == 0x80000u && (keep & 1u))) keep++;
-        int32_t e = exp;
-        if (keep == 16u) { keep >>= 1; e++; }
-        if (e > 8) { keep = 14u; e = 8; }
-        return (sign << 7) | ((uint32_t)(e + 7) << 3) | (keep & 7u);
-    }
-    if (exp < -10) return sign << 7;
-    int32_t sh = 14 - exp;
-    uint32_t mm = m24 >> sh;
-    uint32_t rem = m24 & ((1u << sh) - 1u);
-    uint32_t half = 1u << (sh - 1);
-    if (rem > half || (rem == half && (mm & 1u))) mm++;
-    return (sign << 7) | mm;
-}
-
 // One wave per (row, block): amax by wave reduction, then each lane encodes
 // block/64 elements.  scale = amax/448, 1 for an all-zero block.
 template <int DIM, int BLOCK>

@@ -201,3 +201,205 @@ int launch_gqa_prepare(const float *q_proj, int64_t q_head_stride, const float *
 }
 
 }  // namespace cwick
+
+// ---------------------------------------------------------------------------
+// indexer key production, candidate blocks, dequantised read-back
+// ---------------------------------------------------------------------------
+namespace cwick {
+namespace {
+
+// One wave per closed pool (src/attention.c:486-525): layer-norm statistics of each of the kp
+// raw key rows, a softmax over the pool slots of gate + position bias per dimension, the affine
+// k_norm on the normalised rows, the weighted mean as the pool's key; then the row is quantised
+// like every indexer key (one fp32 scale per row, amax / 448).  hd = 128: two dims per lane.
+__global__ void __launch_bounds__(256)
+ikeys_pool_kernel(const float *__restrict__ tail_k, const float *__restrict__ tail_g, const uint16_t *__restrict__ ape,
+                  const float *__restrict__ knw, const float *__restrict__ knb, float eps, int kp, int64_t n_pools,
+                  uint8_t *__restrict__ out_rows, float *__restrict__ out_scales, float *__restrict__ out_f32) {
+    constexpr int HD = CWICK_HIP_INDEX_DIM;
+    const int lane = threadIdx.x & 63;
+    const int64_t pool = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pool >= n_pools) return;
+    const float *k = tail_k + (size_t)pool * kp * HD, *gt = tail_g + (size_t)pool * kp * HD;
+    // statistics in double like the reference's (sums of 128 floats are exact there in all but
+    // contrived rows, so the order of the wave reduction does not show)
+    float mean[8], inv[8], kv[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        mean[i] = inv[i] = kv[i][0] = kv[i][1] = 0.0f;
+        if (i < kp) {
+            kv[i][0] = k[i * HD + lane];
+            kv[i][1] = k[i * HD + 64 + lane];
+            mean[i] = (float)(wave_sum((double)kv[i][0] + (double)kv[i][1]) / (double)HD);
+            const double t0 = (double)kv[i][0] - (double)mean[i], t1 = (double)kv[i][1] - (double)mean[i];
+            inv[i] = 1.0f / sqrtf((float)(wave_sum(t0 * t0 + t1 * t1) / (double)HD) + eps);
+        }
+    }
+    float res[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int d = lane + 64 * h;
+        float lg[8], mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            lg[i] = -INFINITY;
+            if (i < kp) {
+                lg[i] = gt[i * HD + d] + bf16_to_f32(ape[i * HD + d]);
+                mx = lg[i] > mx ? lg[i] : mx;
+            }
+        }
+        float den = 0.0f, acc = 0.0f;
+        const float w = knw[d], bb = knb[d];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (i < kp) {
+                const float p = expf(lg[i] - mx);
+                den += p;
+                const float nv = ((kv[i][h] - mean[i]) * inv[i]) * w + bb;
+                acc += p * nv;
+            }
+        }
+        res[h] = den > 0.0f ? acc / den : 0.0f;
+    }
+    if (out_f32) {
+        out_f32[(size_t)pool * HD + lane] = res[0];
+        out_f32[(size_t)pool * HD + 64 + lane] = res[1];
+    }
+    const float amax = wave_max(fmaxf(fabsf(res[0]), fabsf(res[1])));
+    const float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+    if (lane == 0) out_scales[pool] = s;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        float v = res[h] / s;
+        v = fminf(fmaxf(v, -448.0f), 448.0f);
+        out_rows[(size_t)pool * HD + lane + 64 * h] = (uint8_t)f32_to_e4m3_rne(v);
+    }
+}
+
+// block maxima of the scores, the partly filled last block forced in (src/ds_model.c:1127-1135)
+__global__ void __launch_bounds__(256)
+cand_blockmax_kernel(const float *__restrict__ scores, int64_t n, int bs, int64_t nblk, float *__restrict__ bsc) {
+    const int lane = threadIdx.x & 63;
+    const int64_t b = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row = blockIdx.y;
+    if (b >= nblk) return;
+    const float *s = scores + (size_t)row * n;
+    const int64_t lo = b * bs, hi = lo + bs < n ? lo + bs : n;
+    float mx = -INFINITY;
+    for (int64_t t = lo + lane; t < hi; t += 64) mx = s[t] > mx ? s[t] : mx;
+    mx = wave_max(mx);
+    if (lane == 0) bsc[(size_t)row * nblk + b] = b == nblk - 1 ? INFINITY : mx;
+}
+
+__global__ void __launch_bounds__(256)
+cand_mark_kernel(const int32_t *__restrict__ blk, int64_t k, int64_t n, int bs, uint8_t *__restrict__ cand) {
+    const int row = blockIdx.y;
+    const int64_t i = (int64_t)blockIdx.x;                 // one workgroup per chosen block
+    if (i >= k) return;
+    const int32_t b = blk[(size_t)row * k + i];
+    if (b < 0) return;
+    const int64_t lo = (int64_t)b * bs, hi = lo + bs < n ? lo + bs : n;
+    for (int64_t t = lo + threadIdx.x; t < hi; t += 256) cand[(size_t)row * n + t] = 1;
+}
+
+__global__ void __launch_bounds__(256) cand_clear_kernel(uint8_t *__restrict__ cand, int64_t total) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < total; i += stride) cand[i] = 0;
+}
+
+// positions outside the candidate blocks cannot be selected (src/ds_model.c:1144-1147)
+__global__ void __launch_bounds__(256)
+cand_apply_kernel(float *__restrict__ scores, const uint8_t *__restrict__ cand, int64_t total) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < total; i += stride)
+        if (!cand[i]) scores[i] = -INFINITY;
+}
+
+template <int DIM, int BLOCK>
+__global__ void __launch_bounds__(256)
+dequant_rows_kernel(const uint8_t *__restrict__ rows, const float *__restrict__ scales, int64_t n, float *__restrict__ out) {
+    constexpr int NBLK = (DIM + BLOCK - 1) / BLOCK;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256, total = n * DIM;
+    for (; i < total; i += stride) {
+        const int64_t r = i / DIM;
+        const int d = (int)(i % DIM);
+        out[i] = e4m3x2_to_f32<false>((uint32_t)rows[i])[0] * scales[r * NBLK + d / BLOCK];
+    }
+}
+
+}  // namespace
+
+int launch_ikeys_pool(const float *tail_k, const float *tail_g, const uint16_t *ape, const float *knw, const float *knb,
+                      float eps, int kpool, int64_t n_pools, uint8_t *out_rows, float *out_scales, float *out_f32,
+                      hipStream_t s) {
+    CWICK_REQUIRE(tail_k && tail_g && ape && knw && knb && out_rows && out_scales, "ikeys_pool: null pointer");
+    CWICK_REQUIRE(kpool >= 1 && kpool <= 8, "ikeys_pool: kpool %d (1..8, src/attention.c:492)", kpool);
+    CWICK_REQUIRE(n_pools >= 1 && n_pools <= ((int64_t)1 << 30), "ikeys_pool: n_pools %lld", (long long)n_pools);
+    ikeys_pool_kernel<<<dim3((unsigned)((n_pools + 3) / 4)), 256, 0, s>>>(tail_k, tail_g, ape, knw, knb, eps, kpool,
+                                                                        n_pools, out_rows, out_scales, out_f32);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_candidate_select(const float *scores, int batch, int64_t n, int block, int64_t topk_blocks, uint8_t *cand,
+                            hipStream_t s) {
+    CWICK_REQUIRE(scores && cand, "candidate_select: null pointer");
+    CWICK_REQUIRE(batch >= 1 && batch <= 65535 && n >= 1 && n <= ((int64_t)1 << 30), "candidate_select: batch %d n %lld",
+                  batch, (long long)n);
+    CWICK_REQUIRE(block >= 1 && topk_blocks >= 1 && topk_blocks <= 65536, "candidate_select: block %d, blocks kept %lld",
+                  block, (long long)topk_blocks);
+    const int64_t nblk = (n + block - 1) / block;
+    // rows this short are selected by the one-workgroup top-k kernels, which take no workspace:
+    // the block scores can sit in this call's
+    CWICK_REQUIRE(nblk < 16384, "candidate_select: %lld blocks (at most 16383)", (long long)nblk);
+    const size_t bsc_b = ((size_t)batch * nblk * 4 + 255) & ~(size_t)255;
+    char *ws = (char *)workspace(s, bsc_b + (size_t)batch * topk_blocks * 4);
+    CWICK_REQUIRE(ws, "candidate_select: workspace allocation failed");
+    float *bsc = (float *)ws;
+    int32_t *blk = (int32_t *)(ws + bsc_b);
+    cand_blockmax_kernel<<<dim3((unsigned)((nblk + 3) / 4), batch), 256, 0, s>>>(scores, n, block, nblk, bsc);
+    CWICK_HIP_CALL(hipGetLastError());
+    {
+        const int64_t total = (int64_t)batch * n;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 8192) blocks = 8192;
+        cand_clear_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(cand, total);      // a kernel, not a memset: safe under graph capture
+    }
+    if (!launch_topk(bsc, batch, nblk, topk_blocks, blk, s)) return 0;
+    cand_mark_kernel<<<dim3((unsigned)topk_blocks, batch), 256, 0, s>>>(blk, topk_blocks, n, block, cand);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_candidate_apply(float *scores, const uint8_t *cand, int batch, int64_t n, hipStream_t s) {
+    CWICK_REQUIRE(scores && cand && batch >= 1 && n >= 1, "candidate_apply: bad argument");
+    const int64_t total = (int64_t)batch * n;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    cand_apply_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(scores, cand, total);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_dequant_latent(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s) {
+    CWICK_REQUIRE(rows && scales && out && n > 0, "dequant_latent: bad argument");
+    int64_t blocks = (n * CWICK_HIP_LATENT_KDIM + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    dequant_rows_kernel<CWICK_HIP_LATENT_KDIM, CWICK_HIP_LATENT_BLOCK><<<dim3((unsigned)blocks), 256, 0, s>>>(rows, scales, n, out);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+int launch_dequant_ikeys(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s) {
+    CWICK_REQUIRE(rows && scales && out && n > 0, "dequant_ikeys: bad argument");
+    int64_t blocks = (n * CWICK_HIP_INDEX_DIM + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    dequant_rows_kernel<CWICK_HIP_INDEX_DIM, CWICK_HIP_INDEX_DIM><<<dim3((unsigned)blocks), 256, 0, s>>>(rows, scales, n, out);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+}  // namespace cwick

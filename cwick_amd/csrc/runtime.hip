@@ -1018,6 +1018,59 @@ int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const 
                               (hipStream_t)stream);
 }
 
+int cwick_hip_ikeys_pool_append_dev(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n, const float *raw_k,
+                                    const float *raw_gate, const uint16_t *ape, const float *k_norm_w,
+                                    const float *k_norm_b, float eps, int kpool, float *rows_f32, void *stream) {
+    clear_error();
+    LATENT_RANGE_CHECK("ikeys_pool_append");
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    return launch_ikeys_pool(raw_k, raw_gate, ape, k_norm_w, k_norm_b, eps, kpool, n,
+                             c->rows + r0 * CWICK_HIP_INDEX_DIM, c->scales + r0, rows_f32, (hipStream_t)stream);
+}
+
+int cwick_hip_candidate_select_dev(const float *scores, int batch, int64_t n, int block, int64_t keep_blocks,
+                                   uint8_t *cand, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_candidate_select(scores, batch, n, block, keep_blocks, cand, (hipStream_t)stream);
+}
+
+int cwick_hip_candidate_apply_dev(float *scores, const uint8_t *cand, int batch, int64_t n, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_candidate_apply(scores, cand, batch, n, (hipStream_t)stream);
+}
+
+int cwick_hip_latent_read_f32(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n, float *rows) {
+    clear_error();
+    LATENT_RANGE_CHECK("latent_read_f32");
+    CWICK_REQUIRE(rows, "latent_read_f32: null argument");
+    size_t bytes = (size_t)n * CWICK_HIP_LATENT_KDIM * sizeof(float);
+    Stager st(c->ctx, pad256(bytes));
+    CWICK_REQUIRE(st.ok, "latent_read_f32: staging allocation failed");
+    float *d = st.room<float>(bytes);
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    if (!launch_dequant_latent(c->rows + r0 * CWICK_HIP_LATENT_KDIM, c->scales + r0 * CWICK_HIP_LATENT_NBLK, n, d,
+                               c->ctx.stream))
+        return 0;
+    if (!st.out(rows, d, bytes)) return 0;
+    return st.wait() ? 1 : 0;
+}
+
+int cwick_hip_ikeys_read_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n, float *rows) {
+    clear_error();
+    LATENT_RANGE_CHECK("ikeys_read_f32");
+    CWICK_REQUIRE(rows, "ikeys_read_f32: null argument");
+    size_t bytes = (size_t)n * CWICK_HIP_INDEX_DIM * sizeof(float);
+    Stager st(c->ctx, pad256(bytes));
+    CWICK_REQUIRE(st.ok, "ikeys_read_f32: staging allocation failed");
+    float *d = st.room<float>(bytes);
+    size_t r0 = (size_t)slot * c->capacity + pos0;
+    if (!launch_dequant_ikeys(c->rows + r0 * CWICK_HIP_INDEX_DIM, c->scales + r0, n, d, c->ctx.stream)) return 0;
+    if (!st.out(rows, d, bytes)) return 0;
+    return st.wait() ? 1 : 0;
+}
+
 int cwick_hip_probe_hbm_read(size_t bytes, int reps, double *gbps) {
     clear_error();
     if (!backend_ready()) return 0;   /* the reason is recorded */

@@ -89,6 +89,11 @@ SIGNATURES = {
     "cwick_hip_mla_expand_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _vp]),
     "cwick_hip_gqa_prepare_dev": (_int, [_vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _flt,
                                          _vp, _vp, _int, _vp, _vp, _vp]),
+    "cwick_hip_ikeys_pool_append_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _flt, _int, _vp, _vp]),
+    "cwick_hip_candidate_select_dev": (_int, [_vp, _int, _i64, _int, _i64, _vp, _vp]),
+    "cwick_hip_candidate_apply_dev": (_int, [_vp, _vp, _int, _i64, _vp]),
+    "cwick_hip_latent_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
+    "cwick_hip_ikeys_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
     "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
     "cwick_hip_probe_mfma": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
@@ -238,6 +243,11 @@ class LatentCache:
                                            scales.ctypes.data), "latent_read")
         return rows, scales
 
+    def read_f32(self, slot, pos0, n):
+        rows = np.empty((n, KDIM), np.float32)
+        _check(lib().cwick_hip_latent_read_f32(self.h, slot, pos0, n, rows.ctypes.data), "latent_read_f32")
+        return rows
+
     def rows_dev(self, slot=0):
         return lib().cwick_hip_latent_rows_dev(self.h, slot)
 
@@ -278,6 +288,18 @@ class IndexKeys:
         _check(lib().cwick_hip_ikeys_read(self.h, slot, pos0, n, rows.ctypes.data,
                                           scales.ctypes.data), "ikeys_read")
         return rows, scales
+
+    def read_f32(self, slot, pos0, n):
+        rows = np.empty((n, IDIM), np.float32)
+        _check(lib().cwick_hip_ikeys_read_f32(self.h, slot, pos0, n, rows.ctypes.data), "ikeys_read_f32")
+        return rows
+
+    def pool_append_dev(self, slot, pos0, n, raw_k, raw_gate, ape, k_norm_w, k_norm_b, eps, kpool,
+                        rows_f32=None, stream=None, raw=False):
+        """Device operands (torch tensors): close n pools and store their keys as rows pos0.."""
+        rc = lib().cwick_hip_ikeys_pool_append_dev(self.h, slot, pos0, n, _dp(raw_k), _dp(raw_gate), _dp(ape),
+                                                   _dp(k_norm_w), _dp(k_norm_b), eps, kpool, _dp(rows_f32), stream)
+        return rc if raw else _check(rc, "ikeys_pool_append_dev")
 
     def rows_dev(self, slot=0):
         return lib().cwick_hip_ikeys_rows_dev(self.h, slot)
@@ -506,6 +528,16 @@ def gqa_prepare_dev(q_proj, q_head_stride, k_proj, v_proj, n, pos0, n_heads, n_k
                                          n_heads, n_kv_heads, head_dim, _dp(q_norm), _dp(k_norm), eps,
                                          _dp(rope_cos), _dp(rope_sin), rotary_dim, _dp(q_out), cache.h, stream)
     return rc if raw else _check(rc, "gqa_prepare_dev")
+
+
+def candidate_select_dev(scores, batch, n, block, keep_blocks, cand, stream=None, raw=False):
+    rc = lib().cwick_hip_candidate_select_dev(_dp(scores), batch, n, block, keep_blocks, _dp(cand), stream)
+    return rc if raw else _check(rc, "candidate_select_dev")
+
+
+def candidate_apply_dev(scores, cand, batch, n, stream=None):
+    return _check(lib().cwick_hip_candidate_apply_dev(_dp(scores), _dp(cand), batch, n, stream),
+                  "candidate_apply_dev")
 
 
 # ------------------------------------------------------------------ phase timers

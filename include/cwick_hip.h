@@ -367,6 +367,53 @@ int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const 
                               const float *rope_sin, int rotary_dim, uint16_t *q_out,
                               cwick_hip_kv *cache, void *stream);
 
+/* Replaces the closing of an indexer pool (indexer_absorb, src/attention.c:
+ * 486-525; the two projections in front of it, :481-482, stay the caller's
+ * GEMVs).  For each of n closed pools: layer-norm statistics of each of the
+ * kpool raw key rows (mean and variance over the 128 dims, in double), a
+ * softmax over the pool's slots, per dimension, of gate + position bias
+ * (`ape`, bf16 [kpool][128]), the affine k_norm (weight and bias fp32 [128])
+ * on the normalised rows, and their softmax-weighted mean as the pool's key.
+ * raw_k and raw_gate fp32 [n][kpool][128] (tail_k / tail_g of the reference,
+ * one pool after the other), kpool 1..8 (:492).  The key is quantised like
+ * every row of the index-key store (one fp32 scale per row, amax / 448) and
+ * stored as rows pos0 .. pos0+n of `slot`; rows_f32, if not NULL, also
+ * receives the unquantised keys, fp32 [n][128] (st->pool of the reference). */
+int cwick_hip_ikeys_pool_append_dev(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n,
+                                    const float *raw_k, const float *raw_gate,
+                                    const uint16_t *ape, const float *k_norm_w,
+                                    const float *k_norm_b, float eps, int kpool,
+                                    float *rows_f32, void *stream);
+
+/* Replaces level one of the two-level selection on the layer that is the
+ * candidate source (src/ds_model.c:1125-1144): the maximum score of every
+ * block of `block` positions, the last (partly filled) block forced in with
+ * +inf (:1134-1135), the keep_blocks best blocks (ds_topk_scores, src/ds_ops.c:
+ * 294-338; blocks of equal maximum are taken lowest index first, which is that
+ * routine's choice on tie-free input), and a byte mask cand[batch][n], 1 inside
+ * a kept block and 0 elsewhere.  scores fp32 [batch][n]; at most 16383 blocks
+ * per row. */
+int cwick_hip_candidate_select_dev(const float *scores, int batch, int64_t n, int block,
+                                   int64_t keep_blocks, uint8_t *cand, void *stream);
+
+/* Replaces the masking on the layers that use the candidates (src/ds_model.c:
+ * 1145-1148): scores outside the kept blocks become -inf, in place, before
+ * cwick_hip_topk_dev picks the positions. */
+int cwick_hip_candidate_apply_dev(float *scores, const uint8_t *cand, int batch, int64_t n,
+                                  void *stream);
+
+/* Replace the fp32 copies of a prefix snapshot (cwick_engine_capture_prefix,
+ * src/engine.c:3626-3641 for the latent rows, :3664-3666 for the indexer pool;
+ * the layout is cwick_prefix_state's, src/pfx.h:63-67): rows pos0 .. pos0+n of
+ * `slot` dequantised (byte value x the scale of its block) into host fp32,
+ * [n][576] and [n][128].  Restoring is cwick_hip_latent_write_f32 /
+ * cwick_hip_ikeys_write_f32; a read followed by a write reproduces the stored
+ * bytes, and each scale to within one unit in its last place (448 s / 448
+ * need not round back to s). */
+int cwick_hip_latent_read_f32(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n,
+                              float *rows);
+int cwick_hip_ikeys_read_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t n, float *rows);
+
 /* ---- phase timers ------------------------------------------------------- */
 /* Replace the reference's attention sub-timers (g_attn_*_ns, src/attention.c:1169-1174,
  * read out by src/prof.c:184-196 under CWICK_PROFILE; CWICK_Q35_PROF's

@@ -55,6 +55,14 @@
  *                                      quarter turn, position 0 is the identity), double
  *                                      brute force, norm preserved by the rotation:
  *                                      PARITY UNPINNED against a reference build
+ *   orc_indexer_pool_row               closed forms (one slot: plain layer norm; equal gates:
+ *                                      the mean of the normalised rows; one dominant gate: that
+ *                                      row), invariance to a constant added to the gates,
+ *                                      double brute force: PARITY UNPINNED against a reference
+ *                                      build
+ *   orc_candidate_mask / _apply        brute force in numpy, last block always kept, number of
+ *                                      blocks kept; the block choice is orc_topk_heap's, which
+ *                                      is pinned against oracle/_ref
  *   orc_indexer_scores[_ds]            double brute force, ReLU-before-weight, thread
  *                                      count invariance: PARITY UNPINNED against a
  *                                      reference build
@@ -994,6 +1002,73 @@ ORC_API int64_t orc_topk_quickselect(const float *sc, int64_t n, int64_t want, i
         }
     free(cp);
     return m;
+}
+
+/* src/attention.c:486-525 (indexer_absorb once the pool has closed): one compressed indexer
+ * key from the pool's kp raw key rows and gate rows.  Statistics in double, everything else in
+ * float, in the reference's order. */
+ORC_API void orc_indexer_pool_row(const float *tail_k, const float *tail_g, const uint16_t *ape,
+                                  const float *knw, const float *knb, float eps, int kp, int hd,
+                                  float *dst) {
+    float mean[8], inv[8];
+    for (int i = 0; i < kp; i++) {
+        const float *row = tail_k + (size_t)i * hd;
+        double s = 0.0;
+        for (int d = 0; d < hd; d++) s += (double)row[d];
+        mean[i] = (float)(s / (double)hd);
+        double v = 0.0;
+        for (int d = 0; d < hd; d++) {
+            double t = (double)row[d] - (double)mean[i];
+            v += t * t;
+        }
+        inv[i] = 1.0f / sqrtf((float)(v / (double)hd) + eps);
+    }
+    for (int d = 0; d < hd; d++) {
+        float mx = -INFINITY;
+        for (int i = 0; i < kp; i++) {
+            float lg = tail_g[(size_t)i * hd + d] + orc_bf16_to_f32(ape[(size_t)i * hd + d]);
+            if (lg > mx) mx = lg;
+        }
+        float den = 0.0f, acc = 0.0f;
+        for (int i = 0; i < kp; i++) {
+            float lg = tail_g[(size_t)i * hd + d] + orc_bf16_to_f32(ape[(size_t)i * hd + d]);
+            float p = expf(lg - mx);
+            den += p;
+            float nv = ((tail_k[(size_t)i * hd + d] - mean[i]) * inv[i]) * knw[d] + knb[d];
+            acc += p * nv;
+        }
+        dst[d] = den > 0.0f ? acc / den : 0.0f;
+    }
+}
+
+/* src/ds_model.c:1125-1144: level one of the two-level selection.  Block maxima, the partly
+ * filled last block forced in, the `keep` best blocks by the reference's heap selector, and a
+ * byte per position.  Returns the number of blocks kept. */
+ORC_API int orc_candidate_mask(const float *scores, int nvis, int bs, int keep, uint8_t *cand) {
+    const int nblk = (nvis + bs - 1) / bs;
+    float *bsc = malloc(sizeof(float) * (size_t)nblk);
+    int *blk = malloc(sizeof(int) * (size_t)(keep > 0 ? keep : 1));
+    for (int b = 0; b < nblk; b++) {
+        int hi = (b + 1) * bs; if (hi > nvis) hi = nvis;
+        float mx = -INFINITY;
+        for (int t = b * bs; t < hi; t++) if (scores[t] > mx) mx = scores[t];
+        bsc[b] = mx;
+    }
+    bsc[(nvis - 1) / bs] = INFINITY;
+    const int k = orc_topk_heap(bsc, nblk, keep, blk);
+    memset(cand, 0, (size_t)nvis);
+    for (int i = 0; i < k; i++) {
+        int b = blk[i];
+        int hi = (b + 1) * bs; if (hi > nvis) hi = nvis;
+        for (int t = b * bs; t < hi; t++) cand[t] = 1;
+    }
+    free(bsc); free(blk);
+    return k;
+}
+
+/* src/ds_model.c:1145-1148: scores outside the candidate blocks become -inf. */
+ORC_API void orc_candidate_apply(float *scores, const uint8_t *cand, int nvis) {
+    for (int t = 0; t < nvis; t++) if (!cand[t]) scores[t] = -INFINITY;
 }
 
 /* ------------------------------------------------------------------ */

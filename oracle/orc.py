@@ -306,6 +306,34 @@ def gqa_prepare(q_proj, q_head_stride, k_proj, v_proj, pos0, H, KV, HD, q_norm, 
     return qo, ko, vo
 
 
+def indexer_pool_row(tail_k, tail_g, ape_bf16, knw, knb, eps):
+    """One compressed indexer key from a closed pool: tail_k, tail_g fp32 [kp][hd], ape bf16 bits."""
+    tail_k = np.ascontiguousarray(tail_k, np.float32)
+    tail_g = np.ascontiguousarray(tail_g, np.float32)
+    ape = np.ascontiguousarray(ape_bf16, np.uint16)
+    kp, hd = tail_k.shape
+    out = np.empty(hd, np.float32)
+    lib().orc_indexer_pool_row(_p(tail_k, C.c_float), _p(tail_g, C.c_float), _p(ape, C.c_uint16),
+                               _p(np.ascontiguousarray(knw, np.float32), C.c_float),
+                               _p(np.ascontiguousarray(knb, np.float32), C.c_float), C.c_float(eps), kp, hd,
+                               _p(out, C.c_float))
+    return out
+
+
+def candidate_mask(scores, block, keep):
+    sc = np.ascontiguousarray(scores, np.float32)
+    cand = np.empty(sc.size, np.uint8)
+    k = lib().orc_candidate_mask(_p(sc, C.c_float), int(sc.size), int(block), int(keep), _p(cand, C.c_uint8))
+    return cand, int(k)
+
+
+def candidate_apply(scores, cand):
+    sc = np.array(scores, np.float32, copy=True)
+    cd = np.ascontiguousarray(cand, np.uint8)
+    lib().orc_candidate_apply(_p(sc, C.c_float), _p(cd, C.c_uint8), int(sc.size))
+    return sc
+
+
 def topk_contract(sc, k):
     sc = np.ascontiguousarray(sc, np.float32)
     out = np.empty(max(min(k, sc.size), 1), np.int32)

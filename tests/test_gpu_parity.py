@@ -841,3 +841,143 @@ def test_gqa_prepare_on_device_then_attention(hip, orc, n, pos0, H, KV, HD, rota
                              rotary, d_q, cache, s, raw=True)
     assert rc == 0 and "capacity" in hip.last_error()
     cache.free()
+
+
+# ------------------------------------------------------------------ indexer pool, candidate blocks, snapshots
+@pytest.mark.parametrize("kp,n_pools", [(4, 301), (1, 5), (8, 64), (3, 2)])
+def test_ikeys_pool_append_on_device(hip, orc, kp, n_pools):
+    """Closing indexer pools on the device (src/attention.c:486-525): the fp32 keys against the
+    oracle's (statistics in double on both sides; expf differs between the device's and the
+    host's library, so 1e-5 relative + 1e-6 absolute, stated), and the stored rows bit for bit
+    against the oracle's quantiser run over the device's own fp32 keys."""
+    import torch
+    say("[case] ikeys_pool_append", kp, n_pools)
+    g = synth.rng(700 + kp)
+    eps = 1e-6
+    tk = (g.standard_normal((n_pools, kp, synth.IDIM), dtype=np.float32) * np.float32(2) + np.float32(0.7))
+    tg = g.standard_normal((n_pools, kp, synth.IDIM), dtype=np.float32)
+    tk[0, 0] = 3.0                                            # a constant row: zero variance, eps carries it
+    ape = synth.f32_to_bf16(g.standard_normal((kp, synth.IDIM), dtype=np.float32) * np.float32(0.5))
+    w = (1 + 0.1 * g.standard_normal(synth.IDIM, dtype=np.float32)).astype(np.float32)
+    b = (0.1 * g.standard_normal(synth.IDIM, dtype=np.float32)).astype(np.float32)
+    c = hip.IndexKeys(2, 512)
+    d = lambda a: torch.from_numpy(a).cuda()
+    d_f32 = torch.empty((n_pools, synth.IDIM), dtype=torch.float32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    c.pool_append_dev(1, 7, n_pools, d(tk), d(tg), d(ape.view(np.int16)), d(w), d(b), eps, kp, d_f32, s)
+    torch.cuda.synchronize()
+    got = d_f32.cpu().numpy()
+    ref = np.stack([orc.indexer_pool_row(tk[i], tg[i], ape, w, b, eps) for i in range(n_pools)])
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+    rows, scales = c.read(1, 7, n_pools)
+    rq, rs = orc.quantize_rows_e4m3(got, synth.IDIM)
+    assert np.array_equal(rows, rq) and np.array_equal(scales.view(np.uint32), rs[:, 0].view(np.uint32))
+    # against the quantised oracle keys: the same bytes but for values that sit on a rounding edge
+    oq, _ = orc.quantize_rows_e4m3(ref, synth.IDIM)
+    assert (rows != oq).mean() < 2e-3
+    # without the fp32 copy, and declined outside the store
+    c.pool_append_dev(0, 0, n_pools, d(tk), d(tg), d(ape.view(np.int16)), d(w), d(b), eps, kp, None, s)
+    torch.cuda.synchronize()
+    r0, s0 = c.read(0, 0, n_pools)
+    assert np.array_equal(r0, rows) and np.array_equal(s0, scales)
+    rc = c.pool_append_dev(0, 512 - n_pools + 1, n_pools, d(tk), d(tg), d(ape.view(np.int16)), d(w), d(b), eps, kp,
+                           None, s, raw=True)
+    assert rc == 0 and "capacity" in hip.last_error()
+    rc = c.pool_append_dev(0, 0, n_pools, d(tk), d(tg), d(ape.view(np.int16)), d(w), d(b), eps, 9, None, s, raw=True)
+    assert rc == 0 and "kpool" in hip.last_error()
+    c.free()
+
+
+@pytest.mark.parametrize("batch,n,bs,keep", [(1, 65536, 64, 32), (4, 10000, 128, 8), (2, 65, 64, 1), (3, 300, 7, 50),
+                                             (1, 5, 64, 3), (2, 131072, 64, 512)])
+def test_candidate_blocks_on_device(hip, orc, batch, n, bs, keep):
+    """Level one of the two-level selection (src/ds_model.c:1125-1148): the byte mask bit for bit
+    against the oracle's, then masked scores -> top-k equal to the oracle's selection over its own
+    masked scores."""
+    import torch
+    say("[case] candidate blocks", batch, n, bs, keep)
+    g = synth.rng(n + bs)
+    sc = g.standard_normal((batch, n), dtype=np.float32)
+    d_sc = torch.from_numpy(sc).cuda()
+    d_cand = torch.full((batch, n), 7, dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.candidate_select_dev(d_sc, batch, n, bs, keep, d_cand, s)
+    torch.cuda.synchronize()
+    cand = d_cand.cpu().numpy()
+    for r in range(batch):
+        want, k = orc.candidate_mask(sc[r], bs, keep)
+        assert np.array_equal(cand[r], want), "row %d" % r
+    # a later layer: its own scores, masked by the shared candidates, then the positions
+    sc2 = g.standard_normal((batch, n), dtype=np.float32)
+    d_sc2 = torch.from_numpy(sc2).cuda()
+    hip.candidate_apply_dev(d_sc2, d_cand, batch, n, s)
+    torch.cuda.synchronize()
+    masked = d_sc2.cpu().numpy()
+    kk = min(n, 2048)
+    d_idx = torch.empty((batch, kk), dtype=torch.int32, device="cuda")
+    hip.topk_dev(d_sc2, batch, n, kk, d_idx, s)
+    torch.cuda.synchronize()
+    idx = d_idx.cpu().numpy()
+    for r in range(batch):
+        ref_masked = orc.candidate_apply(sc2[r], cand[r])
+        assert np.array_equal(masked[r].view(np.uint32), ref_masked.view(np.uint32))
+        n_cand = int(cand[r].sum())
+        # the reference selects `cnt` positions and the -inf ones can only come last; positions
+        # that are candidates fill the list first
+        want = orc.topk_contract(ref_masked, kk)
+        got = idx[r][idx[r] >= 0]
+        if n_cand >= kk:
+            assert np.array_equal(np.sort(got), np.sort(want))
+            assert cand[r][got].all()
+        else:
+            assert cand[r][got].sum() == n_cand
+    rc = hip.candidate_select_dev(d_sc, batch, n, 0, keep, d_cand, s, raw=True)
+    assert rc == 0 and "block" in hip.last_error()
+
+
+def test_candidate_select_declines_too_many_blocks(hip):
+    import torch
+    say("[case] candidate blocks: too many blocks")
+    sc = torch.zeros((1, 20000), dtype=torch.float32, device="cuda")
+    cand = torch.zeros((1, 20000), dtype=torch.uint8, device="cuda")
+    rc = hip.candidate_select_dev(sc, 1, 20000, 1, 4, cand, torch.cuda.current_stream().cuda_stream, raw=True)
+    assert rc == 0 and "16383" in hip.last_error()
+
+
+def test_snapshot_reads_dequantised_rows_and_restores_them(hip, orc):
+    """Prefix snapshots hold fp32 (src/pfx.h:63-67, filled by src/engine.c:3626-3666): rows read
+    back dequantised equal byte value x block scale exactly; writing them into another store
+    reproduces the bytes, and the scales to one unit in the last place; attention over the
+    restored store equals attention over the original."""
+    say("[case] snapshot read_f32 / restore")
+    c3 = synth.cfg3_mla_decode(700, 16, seed=77)
+    lat = hip.LatentCache(2, 1024)
+    lat.write(1, 5, c3["rows"], c3["scales"])
+    f = lat.read_f32(1, 5, 700)
+    lut = orc.e4m3_lut()
+    want = lut[c3["rows"]] * np.repeat(c3["scales"], 128, axis=1)[:, :synth.KDIM]
+    assert np.array_equal(f.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    lat2 = hip.LatentCache(1, 700)
+    lat2.write_f32(0, 0, f)
+    r2, s2 = lat2.read(0, 0, 700)
+    assert np.array_equal(r2, c3["rows"])
+    assert np.abs(s2.view(np.int32) - c3["scales"].view(np.int32)).max() <= 1
+    a = hip.mla_decode(lat, 1, c3["q"], c3["scale"], sel=np.arange(5, 705, dtype=np.int32))
+    b = hip.mla_decode(lat2, 0, c3["q"], c3["scale"], n_list=700)
+    assert_close(b, a, "attention over the restored latent store")
+    # indexer keys
+    g = synth.rng(78)
+    x = g.standard_normal((300, synth.IDIM), dtype=np.float32)
+    x[9] = 0.0
+    ik = hip.IndexKeys(1, 512)
+    ik.write_f32(0, 100, x)
+    rows, scales = ik.read(0, 100, 300)
+    fx = ik.read_f32(0, 100, 300)
+    assert np.array_equal(fx.view(np.uint32), (lut[rows] * scales[:, None]).astype(np.float32).view(np.uint32))
+    ik2 = hip.IndexKeys(1, 300)
+    ik2.write_f32(0, 0, fx)
+    rr, ss = ik2.read(0, 0, 300)
+    assert np.array_equal(rr, rows) and np.abs(ss.view(np.int32) - scales.view(np.int32)).max() <= 1
+    rc = hip.lib().cwick_hip_latent_read_f32(lat.h, 1, 1000, 100, f.ctypes.data)
+    assert rc == 0 and "capacity" in hip.last_error()
+    lat.free(); lat2.free(); ik.free(); ik2.free()

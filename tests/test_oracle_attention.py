@@ -361,3 +361,80 @@ def test_gqa_prepare_closed_forms_and_brute_force(orc):
     y = x[0, 0] / np.sqrt((x[0, 0] ** 2).mean())
     want = y.copy(); want[:rotary // 2] = -y[rotary // 2:rotary]; want[rotary // 2:rotary] = y[:rotary // 2]
     assert np.abs(synth.bf16_to_f32(q2[0, 0]) - want).max() < 2.0 ** -7 * np.abs(want).max()
+
+
+# ------------------------------------------------------------------ indexer pool, candidate blocks
+def _pool_inputs(rng, kp, hd=128):
+    k = (rng.standard_normal((kp, hd)) * 2 + 0.7).astype(np.float32)
+    g = rng.standard_normal((kp, hd)).astype(np.float32)
+    ape = synth.f32_to_bf16(rng.standard_normal((kp, hd)).astype(np.float32) * 0.5)
+    w = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(hd)).astype(np.float32)
+    return k, g, ape, w, b
+
+
+def _layer_norm64(k, w, b, eps):
+    k = k.astype(np.float64)
+    mu = k.mean(axis=-1, keepdims=True)
+    var = ((k - mu) ** 2).mean(axis=-1, keepdims=True)
+    return (k - mu) / np.sqrt(var + eps) * w + b
+
+
+@pytest.mark.parametrize("kp", [1, 3, 4, 8])
+def test_indexer_pool_row_closed_forms_and_brute_force(orc, kp):
+    rng = np.random.default_rng(90 + kp)
+    eps = 1e-6
+    k, g, ape, w, b = _pool_inputs(rng, kp)
+    got = orc.indexer_pool_row(k, g, ape, w, b, eps)
+    normed = _layer_norm64(k, w, b, eps)                                   # [kp, hd]
+    p = softmax64(g.astype(np.float64) + f32(ape), axis=0)                  # over the pool's slots
+    want = (p * normed).sum(axis=0)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+    # a slot-transposed gate or a softmax over the wrong axis would pass none of these:
+    # equal gates and no position bias -> the plain mean of the normalised rows
+    z = np.zeros_like(ape)
+    np.testing.assert_allclose(orc.indexer_pool_row(k, np.zeros_like(g), z, w, b, eps), normed.mean(axis=0),
+                               rtol=2e-5, atol=2e-6)
+    # one slot's gate far above the rest -> that slot's normalised row
+    g1 = np.zeros_like(g)
+    g1[kp - 1] = 60.0
+    np.testing.assert_allclose(orc.indexer_pool_row(k, g1, z, w, b, eps), normed[kp - 1], rtol=2e-5, atol=2e-6)
+    # the same through the position bias alone (60 is exact in bf16)
+    a1 = synth.f32_to_bf16(g1)
+    np.testing.assert_allclose(orc.indexer_pool_row(k, np.zeros_like(g), a1, w, b, eps), normed[kp - 1],
+                               rtol=2e-5, atol=2e-6)
+    # a constant added to every gate of a dimension changes nothing
+    shift = rng.standard_normal((1, 128)).astype(np.float32)
+    np.testing.assert_allclose(orc.indexer_pool_row(k, g + shift, ape, w, b, eps), got, rtol=1e-5, atol=1e-6)
+    if kp == 1:
+        np.testing.assert_allclose(got, normed[0], rtol=2e-5, atol=2e-6)
+
+
+def _brute_candidates(sc, bs, keep):
+    n = sc.size
+    nblk = -(-n // bs)
+    bmax = np.array([sc[b * bs:(b + 1) * bs].max() for b in range(nblk)], np.float64)
+    bmax[(n - 1) // bs] = np.inf
+    order = sorted(range(nblk), key=lambda b: (-bmax[b], b))[:keep]
+    cand = np.zeros(n, np.uint8)
+    for b in order:
+        cand[b * bs:(b + 1) * bs] = 1
+    return cand, len(order)
+
+
+@pytest.mark.parametrize("n,bs,keep", [(1000, 64, 4), (64, 64, 4), (65, 64, 1), (4096, 128, 8), (300, 7, 50), (5, 64, 3)])
+def test_candidate_mask_vs_brute_force(orc, n, bs, keep):
+    rng = np.random.default_rng(n * 31 + bs)
+    sc = rng.standard_normal(n).astype(np.float32)
+    cand, k = orc.candidate_mask(sc, bs, keep)
+    want, wk = _brute_candidates(sc, bs, keep)
+    assert k == wk == min(keep, -(-n // bs))
+    assert np.array_equal(cand, want)
+    assert cand[n - 1] == 1                                    # the partly filled block is always kept
+    assert cand.sum() <= keep * bs
+    masked = orc.candidate_apply(sc, cand)
+    assert np.array_equal(masked[cand == 1], sc[cand == 1])
+    assert np.all(np.isneginf(masked[cand == 0]))
+    # the best position overall survives whenever a block besides the last may be kept
+    if keep >= 2:
+        assert cand[int(np.argmax(sc))] == 1
