@@ -210,7 +210,7 @@ def bench_cfg3(hip, synth, orc, T, stream, a):
     alg = 32768 * (576 + 20) + 128 * 576 * 2 + 128 * 512 * 4
     flops = 2 * 128 * 32768 * (576 + 512)
     t = kern["mla_roles_kernel"]["avg_us"] * 1e-6
-    traffic = profile_traffic("mla_decode_cfg3_pmc_traffic.txt")
+    traffic = profile_traffic("hot_kernels_pmc_traffic.txt")
     r = {"workload": "cfg3 MLA absorbed-latent decode, 128 heads, 32768 x 576 FP8-E4M3 latent "
                      "+ 5 fp32 block scales/token, bf16 q",
          "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern, "alg_bytes": alg, "flops": flops,

@@ -38,12 +38,17 @@
 //   about 3 000 cycles against 1 088 of matrix-core work.  Leaving out the tile copies, the score
 //   MFMAs or the value MFMAs with their conversions takes about a quarter off each, all three
 //   together two thirds; what remains (barrier, exchange, softmax, weights) is the last third.
-//   No single unit is saturated: vector ALU 56 % busy, matrix core 37 %, LDS 32 %.  The copy path
-//   of a compute unit moves a 38 KB tile in about 2 000 cycles when nothing else runs (18 bytes
-//   per cycle, the same from L2-resident rows, with contiguous instead of per-row accesses, and
-//   with loads staged through registers), so 32 query rows per tile cannot reach the matrix
-//   roof; 64 would halve the copies and the conversions per flop.  Eight or sixteen waves per
-//   workgroup (the same work split differently) were measured and are no faster.
+//   No single unit is saturated: vector ALU 56 % busy, matrix core 37 %, LDS 32 %.  A copy
+//   instruction here has one lane per row (64 cache lines touched); alone on the machine that
+//   pattern moves 54 bytes per ns and compute unit from L2 and 18 from HBM, a pattern that walks
+//   along the rows 125 and 25.  Inside this kernel it makes no difference: tile layouts filled
+//   sixteen lines per instruction ([16-key block][piece][key]) or row by row were built, pass
+//   parity and run 4 to 7 % slower, because they spend more vector instructions per copy on
+//   addresses, and the vector ALU, not the copy path, is what a step waits for most.  With 32
+//   query rows per tile the per-tile work that does not depend on the rows (copies, scale
+//   handling, conversions of V) is paid per 1 088 matrix cycles; 64 rows would halve it per
+//   flop.  Eight or sixteen waves per workgroup (the same work split differently) were measured
+//   and are no faster.
 //
 //   LDS tile layout [16-byte column][key 0..63][16 B]: the K fragment is two 16-byte reads per
 //   lane, 256 B contiguous per 16 keys; the V^T fragment of 32 keys x 16 dims is one
