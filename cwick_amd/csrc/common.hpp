@@ -125,6 +125,8 @@ int launch_gqa_prepare(const float *q_proj, int64_t q_head_stride, const float *
                        int64_t n, int64_t pos0, int n_heads, int n_kv_heads, int head_dim, const float *q_norm,
                        const float *k_norm, float eps, const float *rope_cos, const float *rope_sin, int rotary_dim,
                        uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, hipStream_t s);
+int launch_mla_prefill_wide(const uint8_t *rows, const float *scales, int64_t pos0, int64_t n, const uint16_t *q,
+                            int n_heads, float scale, float *out, hipStream_t s);
 int launch_ikeys_pool(const float *tail_k, const float *tail_g, const uint16_t *ape, const float *knw, const float *knb,
                       float eps, int kpool, int64_t n_pools, uint8_t *out_rows, float *out_scales, float *out_f32,
                       hipStream_t s);

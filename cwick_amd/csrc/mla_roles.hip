@@ -963,6 +963,13 @@ int launch_mla_prefill(const uint8_t *rows, const float *scales, int64_t pos0, i
     CWICK_REQUIRE(scale > 0.0f && scale < INFINITY, "mla_prefill: scale must be positive");
     CWICK_REQUIRE((uintptr_t)rows % 16 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)out % 16 == 0,
                   "mla_prefill: rows, q and out must be 16-byte aligned");
+    // 64 heads per workgroup when the query has them (mla_prefill64.hip); CWICK_HIP_MLA_PREFILL=roles
+    // keeps the decode kernel's 32
+    static const bool wide = [] {
+        const char *e = getenv("CWICK_HIP_MLA_PREFILL");
+        return !(e && !strcmp(e, "roles"));
+    }();
+    if (wide && n_heads > HW) return launch_mla_prefill_wide(rows, scales, pos0, n, q, n_heads, scale, out, s);
     Params p{};
     p.rows = rows; p.scales = scales; p.row_bstride = 0; p.scale_bstride = 0;
     p.n_rows = pos0 + n; p.sel = nullptr; p.n_list = pos0 + 1; p.list_step = 1;

@@ -218,7 +218,8 @@ def test_mla_decode_sel(hip, orc):
 
 
 # ------------------------------------------------------------------ MLA prefill
-@pytest.mark.parametrize("pos0,n,nh", [(0, 70, 128), (200, 33, 64), (1000, 5, 16)])
+@pytest.mark.parametrize("pos0,n,nh", [(0, 70, 128), (200, 33, 64), (1000, 5, 16), (4000, 20, 128), (63, 130, 96),
+                                       (129, 64, 128), (0, 1, 128)])
 def test_mla_prefill_chunk(hip, orc, pos0, n, nh):
     say("[case] mla_prefill_chunk", pos0, n, nh)
     c = synth.cfg4_mla_prefill(n, pos0, nh, seed=400 + n)
@@ -227,6 +228,42 @@ def test_mla_prefill_chunk(hip, orc, pos0, n, nh):
     got = hip.mla_prefill_chunk(cache, 0, pos0, c["q"], c["scale"])
     ref = orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"], nthreads=0)
     assert_close(got, ref, "mla_prefill pos0 %d n %d heads %d" % (pos0, n, nh), strict=pos0 >= 200)
+    cache.free()
+
+
+@pytest.mark.parametrize("nh,gain", [(128, 6.0), (128, 12.0), (64, 12.0)])
+def test_mla_prefill_chunk_peaked_scores(hip, orc, nh, gain):
+    """Queries scaled up so that the scores spread over tens of log2 units: the softmax reference of
+    a head moves many times along the keys (64 heads per workgroup move it inside the scoring wave,
+    32 reconcile the key blocks a step later), single keys carry whole rows, and both kernels must
+    still agree with the oracle.  (The score error of Q as two E4M3 terms grows with the score: at
+    gain 12 the scores have a standard deviation of 30 log2 units and near-ties of the two best keys
+    are still resolved inside the tolerance; far beyond that they would not be.)"""
+    say("[case] mla_prefill_chunk peaked", nh, gain)
+    pos0, n = 700, 40
+    c = synth.cfg4_mla_prefill(n, pos0, nh, seed=4400 + nh)
+    q = synth.f32_to_bf16(synth.bf16_to_f32(c["q"]) * np.float32(gain))
+    cache = hip.LatentCache(1, pos0 + n)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_prefill_chunk(cache, 0, pos0, q, c["scale"])
+    ref = orc.mla_prefill_chunk(q, c["rows"], c["scales"], pos0, c["scale"], nthreads=0)
+    assert_close(got, ref, "mla_prefill peaked heads %d gain %g" % (nh, gain), strict=False)
+    cache.free()
+
+
+def test_mla_prefill_wide_equals_the_decode_kernel(hip, orc):
+    """The 64-head prefill kernel against the decode kernel run query by query through the same
+    ABI (same operands, two different kernels, both with fp16 weights: up to 6e-4 each against
+    the exact result): the difference between them stays inside the tolerance against the oracle."""
+    say("[case] mla_prefill wide vs decode per query")
+    pos0, n, nh = 300, 9, 128
+    c = synth.cfg4_mla_prefill(n, pos0, nh, seed=4500)
+    cache = hip.LatentCache(1, pos0 + n)
+    cache.write(0, 0, c["rows"], c["scales"])
+    got = hip.mla_prefill_chunk(cache, 0, pos0, c["q"], c["scale"])
+    for t in range(n):
+        one = hip.mla_decode(cache, 0, c["q"][t], c["scale"], n_list=pos0 + t + 1)
+        assert np.abs(got[t] - one).max() <= 1.5e-3, "query %d: %g" % (t, np.abs(got[t] - one).max())
     cache.free()
 
 

@@ -78,7 +78,7 @@ def test_no_valu_write_right_before_an_mfma_reads_it(src):
     assert not early, "MFMA result read before the matrix pipe has written it: %r" % early[:3]
 
 
-LDS_DMA_SOURCES = ["mla_roles.hip", "gqa_prefill.hip"]
+LDS_DMA_SOURCES = ["mla_roles.hip", "mla_prefill64.hip", "gqa_prefill.hip"]
 
 
 @pytest.mark.parametrize("src", LDS_DMA_SOURCES)
