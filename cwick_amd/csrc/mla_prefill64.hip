@@ -21,8 +21,15 @@
 //                v_mfma_f32_16x16x32_f16, every converted V^T fragment used four times.
 //   The roles run one tile apart (tile t+1 is scored while tile t is accumulated): one barrier
 //   per step.  Tile t+2 is copied (global_load_lds, issued from assembly) at the top of step t
-//   into the stage tile t-1 left at the last barrier.
+//   into the stage tile t-1 left at the last barrier, by the value waves alone: a wave stalls
+//   while the memory pipeline takes its copies, and the scoring waves are the longer pole of a
+//   step (copies dealt to all eight waves: 36.1 ms for 4096 queries over 28672 + 4096 rows,
+//   by the value waves: 31.2; spreading them over the step or issuing them a step earlier into
+//   the columns a value wave has just finished with: 31.1 and 34).
 //   One slice per query: no partials, the value waves write the output.
+//   Ablation builds at 31 ms: without the value MFMAs and conversions 21.7, without the score
+//   MFMAs and K reads 22.4, without the K reads alone 27.3: the two roles weigh the same and
+//   mostly add up; the matrix pipe is busy 2 176 of about 4 200 cycles per step and SIMD.
 #include "common.hpp"
 
 #include <cstdlib>
@@ -183,6 +190,21 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
         else dma4(sp + 4 * (wave - 4), tile_off + SC_OFF + (uint32_t)(wave - 4) * (TK * 4));
         if (wave == 0) dma4(sp + 16, tile_off + SC_OFF + 4u * (TK * 4));
     };
+    // a tile by the four value waves alone (the loop: the scoring waves are the longer pole of a
+    // step and a wave stalls while the memory pipeline takes its copies): wave cw copies columns
+    // cw, cw + 4, .. cw + 32, scale block cw, and wave 4 also scale block 4
+    auto share_v = [&](int t, uint32_t tile_off) {
+        const int r = t * TK + lane;
+        const bool live = r < n_keys;
+        const uint64_t rp = live ? (uint64_t)(uintptr_t)rows + (uint64_t)(uint32_t)r * KDIM : zrow;
+        const uint64_t sp = live ? (uint64_t)(uintptr_t)scales + (uint64_t)(uint32_t)r * (NBLK * 4) : zsc;
+        const uint32_t col_off = tile_off + (uint32_t)cw * (TK * 16);
+        const uint64_t col_src = rp + 16 * cw;
+#pragma unroll
+        for (int k = 0; k < 9; k++) dma16(col_src + 64 * k, col_off + (uint32_t)(4 * k) * (TK * 16));
+        dma4(sp + 4 * cw, tile_off + SC_OFF + (uint32_t)cw * (TK * 4));
+        if (cw == 0) dma4(sp + 16, tile_off + SC_OFF + 4u * (TK * 4));
+    };
     if (n_tiles > 0) share(0, lds0);                  // stage 0 is not part of the Q park area
 
     // ---- Q for 4 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
@@ -261,7 +283,8 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
     if (scorer)
         asm volatile("" : "+v"(qhi[0]), "+v"(qhi[1]), "+v"(qhi[2]), "+v"(qhi[3]), "+v"(qlo[0]), "+v"(qlo[1]), "+v"(qlo[2]), "+v"(qlo[3]), "+v"(qrope), "+v"(qsc0), "+v"(qsc1));
 
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0
+    if (n_tiles > 1) share(1, lds0 + TILE_B);         // tiles 0 and 1 are whole when the loops start
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     LDS_BARRIER();
 
     const float c0 = p.scale * 1.44269504088896340736f;   // scores in log2 units
@@ -296,9 +319,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
 
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
-#ifndef P64_ABL_NOCOPY
-            if (t + 2 < n_tiles) share(t + 2, st_cp);     // the stage tile t-1 left at the last barrier
-#endif
             if (t + 1 < n_tiles) {
                 // ---- scores S^T[key][head] for all 64 keys, heads 16 hq.. of tile t+1 ----
                 const uint32_t tb = st_sc;
@@ -315,9 +335,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                         const u32x4 k1 = LDS_AT(lds_u32x4, a + TK * 16);
                         return (i32x8){(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
                     };
-#ifdef P64_ABL_NOQK
-                    S[kb] = LDS_AT(lds_f32x4, sa) * 1e-3f;
-#else
                     i32x8 kA = kfrag(0);
 #pragma unroll
                     for (int b = 0; b < 4; b++) {
@@ -346,7 +363,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                         const f32x4 acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qrope, z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc1);
                         S[kb] += acc * scb;
                     }
-#endif
                     S[kb] *= c0;
                 }
                 // positions past the query's last key (only in its last tile)
@@ -387,8 +403,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 l_priv += lsum;
                 LDS_AT(lds_u32, xn + xf_off) = moves ? 1u : 0u;
             }
-            // this wave's share of tile t+2 has to be whole at the barrier: tile t+2 is scored in the next step
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             LDS_BARRIER();
             rotate();
         }
@@ -420,9 +434,7 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
         asm volatile("" ::: "memory");
 #pragma clang loop unroll(disable)
         for (int t = -1; t < n_tiles; t++) {
-#ifndef P64_ABL_NOCOPY
-            if (t + 2 < n_tiles) share(t + 2, st_cp);     // the stage tile t-1 left at the last barrier
-#endif
+            if (t >= 0 && t + 2 < n_tiles) share_v(t + 2, st_cp);     // the stage tile t-1 left at the last barrier
             if (t >= 0) {
                 // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 64 heads, tile t ----
                 const uint32_t tb = st_val;
@@ -483,7 +495,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                     }
                 }
                 const uint32_t va0 = tb + tr_off;
-#ifndef P64_ABL_NOPV
 #pragma unroll
                 for (int kh = 0; kh < 2; kh++) {
                     u32x4 pw[NHQ];                        // the tile's weights of this key half, per 16-head block
@@ -514,10 +525,8 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                         __builtin_amdgcn_sched_barrier(0);   // the next block's fragments are not fetched across this point (registers)
                     }
                 }
-#else
-                oacc[0][0][0] += __builtin_bit_cast(float, va0 + sw[0][0] + sw[1][1]);
-#endif
             }
+            // tile t+2, copied by the value waves during this step, is scored in the next one
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             LDS_BARRIER();
             rotate();
