@@ -261,7 +261,7 @@ def bench_cfg4(hip, synth, orc, T, stream, a):
     wall, kern, spread = T.run(step)
     keys = n * pos0 + n * (n + 1) // 2
     flops = 2 * nh * (576 + 512) * keys
-    kname = "mla_prefill_kernel" if "mla_prefill_kernel" in kern else "mla_roles_kernel"
+    kname = "mla_prefill64_kernel" if "mla_prefill64_kernel" in kern else "mla_roles_kernel"
     t = kern[kname]["avg_us"] * 1e-6
     r = {"workload": "cfg4 MLA chunked prefill, 4096 queries appended to 28672 FP8 latent rows",
          "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern, "flops": flops,

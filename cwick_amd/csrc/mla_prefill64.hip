@@ -570,7 +570,7 @@ int launch_mla_prefill_wide(const uint8_t *rows, const float *scales, int64_t po
     const int64_t total = (int64_t)n_hb * n;
     CWICK_REQUIRE(total <= 0x7FFFFFFF, "mla_prefill: grid of %lld workgroups is too large", (long long)total);
     {
-        ProfScope ps(CWICK_HIP_PROF_MLA, s);
+        ProfScope ps(CWICK_HIP_PROF_MLA_PREFILL, s);
         mla_prefill64_kernel<<<dim3((unsigned)total), THREADS, smem, s>>>(p);
     }
     CWICK_HIP_CALL(hipGetLastError());

@@ -565,10 +565,12 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
         beta = (other <= beta) ? beta : other;                  // NaN sticks
     }
     if (lane == 0) sh_beta[tid >> 6] = beta;
-    // three digits are enough here: the k-th largest key lies in the bucket [T_lo, T_hi] of the
-    // 24-bit prefix; at most k-1 keys lie above the bucket and at least k in or above it, which
-    // is all the argument needs, and the bucket is 256 ulps wide, far inside beta
-    const TopkMwState st = topk_mw_pick(slices + (size_t)2 * sl * 256, n_wg, 8, state[2], hist, &sh_state);
+    // two digits are enough here: the k-th largest key lies in the bucket [T_lo, T_hi] of the
+    // 16-bit prefix (sign, exponent, seven bits of the fraction); at most k-1 keys lie above the
+    // bucket and at least k in or above it, which is all the argument needs.  The bucket is 2^-7
+    // of the threshold wide, about as much as beta on the indexer's scores: a third digit pass
+    // (5.4 us) would trim the candidate list by a quarter, which costs the rescoring less.
+    const TopkMwState st = topk_mw_pick(slices + (size_t)1 * sl * 256, n_wg, 16, state[1], hist, &sh_state);
     beta = sh_beta[0];
 #pragma unroll
     for (int i = 1; i < TOPK_MW_THREADS / 64; i++) beta = (sh_beta[i] <= beta) ? beta : sh_beta[i];
@@ -576,8 +578,8 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     auto key_float = [](uint32_t key) -> float {
         return __builtin_bit_cast(float, (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
     };
-    const float T_lo = key_float(st.prefix), T_hi = key_float(st.prefix | 0xFFu);
-    const bool ok = (st.prefix >> 8) != 0u && beta >= 0.0f && beta < INFINITY && T_lo == T_lo && T_hi == T_hi;
+    const float T_lo = key_float(st.prefix), T_hi = key_float(st.prefix | 0xFFFFu);
+    const bool ok = (st.prefix >> 16) != 0u && beta >= 0.0f && beta < INFINITY && T_lo == T_lo && T_hi == T_hi;
     if (!ok) {
         if (wg == 0 && tid == 0) rows[row].fallback = 1u;
         return;
@@ -848,7 +850,7 @@ int launch_topk_band_classify(float *scores, int batch, int64_t n, int64_t k, ui
     CWICK_REQUIRE(n_s0 <= 2 * TOPK_MW_MAX_WGS, "topk_band_classify: %d first-digit slices", n_s0);
     const size_t ws_row = topk_mw_band_row_dwords(n);
     const dim3 grid((unsigned)n_wg, (unsigned)batch);
-    for (int pass = digit0_done ? 1 : 0; pass < 3; pass++)
+    for (int pass = digit0_done ? 1 : 0; pass < 2; pass++)
         topk_mw_hist_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, pass, ws, ws_row, sl, n_s0);
     topk_mw_classify_kernel<<<grid, TOPK_MW_THREADS, 0, s>>>(scores, n, k, (int)n_wg, ws, ws_row, beta_slots,
                                                             n_beta, cand, cap, rows, sl, hi_count);

@@ -426,10 +426,11 @@ enum {
     CWICK_HIP_PROF_GQA_DECODE = 0,      /* gqa_decode_split_kernel */
     CWICK_HIP_PROF_GQA_DECODE_MERGE,    /* splitk_merge_wide_kernel<256|128> after it */
     CWICK_HIP_PROF_GQA_PREFILL,         /* gqa_prefill_kernel */
-    CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill) */
+    CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill of at most 64 heads) */
     CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag16_kernel after it */
-    CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel, or in a fused select indexer_approx_kernel + 2 x topk_mw_hist_kernel + topk_mw_classify_kernel + indexer_rescore_kernel + the exact kernel's fallback pass */
+    CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel, or in a fused select indexer_approx_kernel + topk_mw_hist_kernel + topk_mw_classify_kernel + indexer_rescore_kernel + the exact kernel's fallback pass */
     CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel; in a fused select topk_band_finish_kernel */
+    CWICK_HIP_PROF_MLA_PREFILL,         /* mla_prefill64_kernel (chunked prefill of more than 64 heads) */
     CWICK_HIP_PROF_COUNT
 };
 void cwick_hip_prof_enable(int on);
