@@ -34,6 +34,7 @@ int num_cus();
 // asks for more bytes; kernels enqueued earlier on the stream have finished
 // with it by the time a later enqueue on the same stream touches it.
 void *workspace(hipStream_t s, size_t bytes);
+uint32_t *ticket_counters(hipStream_t s);   // 64 dwords per stream, zero between kernels
 
 // Phase timer: brackets the launches made while it is alive with two events on
 // `s` when profiling is enabled; does nothing (and records nothing) otherwise.

@@ -667,27 +667,50 @@ template <int GROUP>
 __global__ void __launch_bounds__(PF_THREADS, 1)
 gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
                    const uint16_t *__restrict__ Q, int64_t pos0, int64_t n, int n_kv_heads,
-                   float scale_log2e, float *__restrict__ out, int64_t n_prec) {
+                   float scale_log2e, float *__restrict__ out, int64_t n_prec, int64_t pblocks,
+                   uint32_t *__restrict__ tickets) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    // Workgroups are handed out in grid order, so the grid runs from the most expensive position
-    // block to the cheapest (the last ones to start must be the short ones).  A block costs its
-    // number of key tiles, and 1.6 times that in the PRECISE variant: rank r = blockIdx.x /
-    // n_kv_heads in the merge of the two descending sequences 10 (p+1), p >= n_prec, and
-    // 16 (p+1), p < n_prec.
-    const int64_t pblocks = (int64_t)gridDim.x / n_kv_heads;
-    const int64_t rank = (int64_t)blockIdx.x / n_kv_heads;
-    const int kvh = (int)(blockIdx.x % n_kv_heads);
-    int64_t pblk = -1, before = 0;                      // precise blocks ranked before this one
-    for (int64_t pp = n_prec - 1; pp >= 0; pp--) {
-        int64_t qmin = 16 * (pp + 1) / 10;              // plain blocks q >= qmin cost more than precise block pp
-        if (qmin < n_prec) qmin = n_prec;
-        const int64_t rk = (qmin < pblocks ? pblocks - qmin : 0) + (n_prec - 1 - pp);
-        if (rk == rank) pblk = pp;
-        if (rk < rank) before++;
+    __shared__ uint32_t sh_item;
+    // One workgroup per compute unit stays for the whole launch and draws its (position block,
+    // kv head) items from a counter: a compute unit that the dispatcher would leave empty for
+    // 4 to 30 us between two workgroups goes on at once, and XCDs that run slower than the others
+    // (two of the eight took 6 % longer for the same share) simply draw fewer items.  Items are
+    // handed out from the most expensive position block to the cheapest (the last ones to start
+    // must be the short ones).  A block costs its number of key tiles, and 1.6 times that in the
+    // PRECISE variant: rank r = item / n_kv_heads in the merge of the two descending sequences
+    // 10 (p+1), p >= n_prec, and 16 (p+1), p < n_prec.
+    const uint32_t total = (uint32_t)(pblocks * n_kv_heads);
+    for (;;) {
+        // nothing of the last item may still be on its way into LDS
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0) sh_item = atomicAdd(&tickets[0], 1u);
+        __syncthreads();
+        const uint32_t item = sh_item;
+        __syncthreads();                                 // everybody has the item, and is done with the last one's LDS
+        if (item >= total) break;
+        const int64_t rank = (int64_t)item / n_kv_heads;
+        const int kvh = (int)(item % (uint32_t)n_kv_heads);
+        int64_t pblk = -1, before = 0;                  // precise blocks ranked before this one
+        for (int64_t pp = n_prec - 1; pp >= 0; pp--) {
+            int64_t qmin = 16 * (pp + 1) / 10;          // plain blocks q >= qmin cost more than precise block pp
+            if (qmin < n_prec) qmin = n_prec;
+            const int64_t rk = (qmin < pblocks ? pblocks - qmin : 0) + (n_prec - 1 - pp);
+            if (rk == rank) pblk = pp;
+            if (rk < rank) before++;
+        }
+        if (pblk < 0) pblk = pblocks - 1 - (rank - before);
+        if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
+        else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
     }
-    if (pblk < 0) pblk = pblocks - 1 - (rank - before);
-    if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
-    else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
+    // the last workgroup to leave puts the counters back to zero for the next launch (every
+    // workgroup has drawn its last ticket before it counts itself out)
+    if (threadIdx.x == 0) {
+        const uint32_t gone = atomicAdd(&tickets[1], 1u);
+        if (gone == gridDim.x - 1) {
+            __hip_atomic_store(&tickets[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&tickets[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 }
 
 // rows that see at most this many keys take the two-term-weight variant
@@ -725,10 +748,14 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
         if (pos0 + last_t + 1 > gqa_precise_keys()) break;
         n_prec++;
     }
+    uint32_t *tickets = ticket_counters(s);
+    CWICK_REQUIRE(tickets, "gqa_prefill: ticket counters");
+    const int64_t items = pblocks * n_kv_heads;
+    const int64_t wgs = items < num_cus() ? items : num_cus();      // the LDS of a compute unit holds one workgroup
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_PREFILL, s);
-        gqa_prefill_kernel<GROUP><<<dim3((unsigned)(pblocks * n_kv_heads)), PF_THREADS, smem, s>>>(
-            k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec);
+        gqa_prefill_kernel<GROUP><<<dim3((unsigned)wgs), PF_THREADS, smem, s>>>(
+            k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec, pblocks, tickets);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

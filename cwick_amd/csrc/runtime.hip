@@ -127,9 +127,31 @@ void *workspace(hipStream_t s, size_t bytes) {
     return grow_one(g_ws[s], s, bytes);
 }
 
+// A few dwords per stream that are zero whenever no kernel of the stream is running: kernels
+// that hand out their work by tickets count in them and leave them zero again.
+static std::unordered_map<hipStream_t, uint32_t *> g_tickets;
+uint32_t *ticket_counters(hipStream_t s) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_tickets.find(s);
+    if (it != g_tickets.end()) return it->second;
+    void *p = nullptr;
+    if (!hip_ok(hipMalloc(&p, 256), "hipMalloc(tickets)")) return nullptr;
+    if (!hip_ok(hipMemset(p, 0, 256), "hipMemset(tickets)")) {
+        (void)hipFree(p);
+        return nullptr;
+    }
+    g_tickets[s] = (uint32_t *)p;
+    return (uint32_t *)p;
+}
+
 // forget (and free) the workspace of a stream that is about to be destroyed
 static void drop_workspace(hipStream_t s) {
     std::lock_guard<std::mutex> lk(g_mu);
+    auto tk = g_tickets.find(s);
+    if (tk != g_tickets.end()) {
+        (void)hipFree(tk->second);
+        g_tickets.erase(tk);
+    }
     auto it = g_ws.find(s);
     if (it == g_ws.end()) return;
     if (it->second.p) (void)hipFree(it->second.p);
@@ -220,6 +242,8 @@ static void free_all_scratch() {
     std::lock_guard<std::mutex> lk(g_mu);
     for (auto &kv : g_ws) if (kv.second.p) (void)hipFree(kv.second.p);
     g_ws.clear();
+    for (auto &kv : g_tickets) (void)hipFree(kv.second);
+    g_tickets.clear();
 }
 
 }  // namespace cwick
