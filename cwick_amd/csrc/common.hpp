@@ -49,7 +49,7 @@ struct ProfScope {
 // ---- kernel launchers (one per .hip file) ----------------------------------
 int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
                       int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
-                      hipStream_t s);
+                      hipStream_t s, const int32_t *sel = nullptr, int64_t n_rows = 0);
 int launch_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, int64_t n,
                        int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
                        float scale, float *out, hipStream_t s);

@@ -17,6 +17,9 @@
 //   broadcast.  Online softmax per lane group, KB rows per step to amortise
 //   the rescale; the lane groups of a workgroup are merged through LDS, then
 //   (m, l, acc) goes to the workspace and a second kernel merges the splits.
+//   With a position list (sel[]: the block-sparse decode of src/mm_model.c:1962-2047, whose
+//   selected blocks the caller has expanded to positions) list entry i names cache row sel[i];
+//   entries that name no row (negative, or beyond n_rows) carry no weight.
 #include "common.hpp"
 #include "merge.hpp"
 
@@ -31,6 +34,7 @@ template <int HD, int GROUP>
 __global__ void __launch_bounds__(GQA_DEC_THREADS)
 gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
                         const uint16_t *__restrict__ Q, int64_t n_keys, int n_kv_heads,
+                        const int32_t *__restrict__ sel, int64_t n_rows,
                         int keys_per_split, float scale,
                         float *__restrict__ part_acc,   // [n_splits][n_heads][HD]
                         float *__restrict__ part_ml) {  // [n_splits][n_heads][2]
@@ -73,10 +77,16 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
     for (int64_t base = k_begin + (int64_t)grp * GQA_DEC_KB; base < k_end;
          base += (int64_t)NGRP * GQA_DEC_KB) {
         u32x4 kw[GQA_DEC_KB], vw[GQA_DEC_KB];
+        bool dead[GQA_DEC_KB];
 #pragma unroll
         for (int r = 0; r < GQA_DEC_KB; r++) {
             // rows past the slice are clamped (their weight is forced to zero below)
             int64_t t = base + r < k_end ? base + r : k_end - 1;
+            dead[r] = base + r >= k_end;
+            if (sel) {
+                t = sel[t];
+                if (t < 0 || t >= n_rows) dead[r] = true, t = 0;
+            }
             kw[r] = *(const u32x4 *)(Kg + t * row_stride);
             vw[r] = *(const u32x4 *)(Vg + t * row_stride);
         }
@@ -106,7 +116,7 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
                 for (int j = 0; j < GROUP; j++) s[r][j] += __shfl_xor(s[r][j], o, 64);
 #pragma unroll
         for (int r = 0; r < GQA_DEC_KB; r++)
-            if (base + r >= k_end)
+            if (dead[r])
 #pragma unroll
                 for (int j = 0; j < GROUP; j++) s[r][j] = -INFINITY;
 
@@ -115,15 +125,15 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
             float mx = m[j];
 #pragma unroll
             for (int r = 0; r < GQA_DEC_KB; r++) mx = fmaxf(mx, s[r][j]);
-            // mx is finite: row `base` itself is always inside the slice
-            const float corr = __expf(m[j] - mx);
+            // all of a step's rows can be dead in a list: then nothing moves (exp(-inf) = 0)
+            const float corr = __expf(m[j] - (mx == -INFINITY ? 0.0f : mx));
             m[j] = mx;
             l[j] *= corr;
 #pragma unroll
             for (int i = 0; i < 8; i++) acc[j][i] *= corr;
 #pragma unroll
             for (int r = 0; r < GQA_DEC_KB; r++) {
-                const float p = __expf(s[r][j] - mx);
+                const float p = __expf(s[r][j] - (mx == -INFINITY ? 0.0f : mx));
                 l[j] += p;
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -196,7 +206,8 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
 
 template <int HD, int GROUP>
 static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
-                          const uint16_t *q, float scale, float *out, hipStream_t s) {
+                          const int32_t *sel, int64_t n_rows, const uint16_t *q, float scale, float *out,
+                          hipStream_t s) {
     const int n_heads = n_kv_heads * GROUP;
     constexpr int LPK = HD / 8, NGRP = GQA_DEC_THREADS / LPK;
     constexpr int step = NGRP * GQA_DEC_KB;   // rows one workgroup consumes per iteration
@@ -219,7 +230,7 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_DECODE, s);
         gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_kv_heads), GQA_DEC_THREADS, 0, s>>>(
-            k, v, q, n_keys, n_kv_heads, (int)per, scale, part_acc, part_ml);
+            k, v, q, n_keys, n_kv_heads, sel, n_rows, (int)per, scale, part_acc, part_ml);
     }
     CWICK_HIP_CALL(hipGetLastError());
     {
@@ -233,7 +244,7 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
 
 int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
                       int head_dim, const uint16_t *q, int n_heads, float scale, float *out,
-                      hipStream_t s) {
+                      hipStream_t s, const int32_t *sel, int64_t n_rows) {
     CWICK_REQUIRE(k && v && q && out, "gqa_decode: null pointer");
     CWICK_REQUIRE(n_keys >= 1 && n_keys <= ((int64_t)1 << 30), "gqa_decode: n_keys %lld",
                   (long long)n_keys);
@@ -245,7 +256,7 @@ int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int 
     const int group = n_heads / n_kv_heads;
 #define CASE(HD, G)                                      \
     if (head_dim == HD && group == G)                    \
-        return run_gqa_decode<HD, G>(k, v, n_keys, n_kv_heads, q, scale, out, s)
+        return run_gqa_decode<HD, G>(k, v, n_keys, n_kv_heads, sel, n_rows, q, scale, out, s)
     CASE(256, 1); CASE(256, 2); CASE(256, 4); CASE(256, 8);
     CASE(128, 1); CASE(128, 2); CASE(128, 4); CASE(128, 8);
 #undef CASE

@@ -755,6 +755,37 @@ int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q, int
     return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
+int cwick_hip_gqa_decode_sel_dev(const uint16_t *k, const uint16_t *v, int64_t n_rows, int n_kv_heads,
+                                 int head_dim, const int32_t *sel, int64_t n_list, const uint16_t *q,
+                                 int n_heads, float scale, float *out, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    CWICK_REQUIRE(sel && n_rows >= 1 && n_rows <= ((int64_t)1 << 31) - 1, "gqa_decode_sel: list or n_rows %lld",
+                  (long long)n_rows);
+    return launch_gqa_decode(k, v, n_list, n_kv_heads, head_dim, q, n_heads, scale, out, (hipStream_t)stream, sel,
+                             n_rows);
+}
+
+int cwick_hip_gqa_decode_sel(cwick_hip_kv *c, const int32_t *sel, int64_t n_list, const uint16_t *q,
+                             int n_heads, float scale, float *out) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    CWICK_REQUIRE(c && sel && q && out, "gqa_decode_sel: null argument");
+    CWICK_REQUIRE(n_list >= 1 && n_list <= ((int64_t)1 << 24), "gqa_decode_sel: n_list %lld", (long long)n_list);
+    CWICK_REQUIRE(n_heads > 0 && n_heads <= 1024, "gqa_decode_sel: n_heads %d", n_heads);
+    size_t qb = (size_t)n_heads * c->head_dim * 2, ob = (size_t)n_heads * c->head_dim * 4, sb = (size_t)n_list * 4;
+    Stager st(c->ctx, pad256(qb) + pad256(ob) + pad256(sb));
+    CWICK_REQUIRE(st.ok, "gqa_decode_sel: staging allocation failed");
+    const uint16_t *dq = st.in(q, qb);
+    const int32_t *dsel = st.in(sel, sb);
+    CWICK_REQUIRE(dq && dsel, "gqa_decode_sel: upload failed");
+    float *dout = st.room<float>(ob);
+    if (!launch_gqa_decode(c->k, c->v, n_list, c->n_kv_heads, c->head_dim, dq, n_heads, scale, dout, c->ctx.stream,
+                           dsel, c->capacity))
+        return 0;
+    return st.out(out, dout, ob) && st.wait() ? 1 : 0;
+}
+
 int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *q, int n_heads,
                           float scale, float *out) {
     clear_error();

@@ -89,6 +89,8 @@ SIGNATURES = {
     "cwick_hip_mla_expand_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _vp]),
     "cwick_hip_gqa_prepare_dev": (_int, [_vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _flt,
                                          _vp, _vp, _int, _vp, _vp, _vp]),
+    "cwick_hip_gqa_decode_sel": (_int, [_vp, _vp, _i64, _vp, _int, _flt, _vp]),
+    "cwick_hip_gqa_decode_sel_dev": (_int, [_vp, _vp, _i64, _int, _int, _vp, _i64, _vp, _int, _flt, _vp, _vp]),
     "cwick_hip_ikeys_pool_append_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _flt, _int, _vp, _vp]),
     "cwick_hip_candidate_select_dev": (_int, [_vp, _int, _i64, _int, _i64, _vp, _vp]),
     "cwick_hip_candidate_apply_dev": (_int, [_vp, _vp, _int, _i64, _vp]),
@@ -325,6 +327,23 @@ def gqa_decode(cache, n_keys, q, scale, raw=False):
         return rc, out
     _check(rc, "gqa_decode")
     return out
+
+
+def gqa_decode_sel(cache, sel, q, scale, raw=False):
+    q, qp = _np(q, np.uint16)
+    sel, sp = _np(sel, np.int32)
+    nh, hd = q.shape
+    out = np.empty((nh, hd), np.float32)
+    rc = lib().cwick_hip_gqa_decode_sel(cache.h, sp, sel.size, qp, nh, scale, out.ctypes.data)
+    if raw:
+        return rc, out
+    _check(rc, "gqa_decode_sel")
+    return out
+
+
+def gqa_decode_sel_dev(k, v, n_rows, n_kv_heads, head_dim, sel, n_list, q, n_heads, scale, out, stream=None):
+    return _check(lib().cwick_hip_gqa_decode_sel_dev(_dp(k), _dp(v), n_rows, n_kv_heads, head_dim, _dp(sel), n_list,
+                                                     _dp(q), n_heads, scale, _dp(out), stream), "gqa_decode_sel_dev")
 
 
 def gqa_prefill(cache, pos0, q, scale, raw=False):

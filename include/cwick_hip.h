@@ -367,6 +367,21 @@ int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const 
                               const float *rope_sin, int rotary_dim, uint16_t *q_out,
                               cwick_hip_kv *cache, void *stream);
 
+/* Replaces the attention of the block-sparse GQA decode (src/mm_model.c:
+ * 1962-2047: per head, scores over the selected positions selpos[] with the
+ * kv head h / group, max, exp, sum, normalise, weighted sum of the V rows).
+ * sel[i] is a cache row; the caller expands its selected blocks
+ * (mm_select_blocks, :1733-1761) into positions as the reference does
+ * (:1966-1973).  Entries that are negative or not below the number of rows
+ * carry no weight; a list without a valid entry gives zeros.  Softmax is a sum:
+ * the order of the list does not matter beyond rounding. */
+int cwick_hip_gqa_decode_sel(cwick_hip_kv *c, const int32_t *sel, int64_t n_list, const uint16_t *q,
+                             int n_heads, float scale, float *out);
+int cwick_hip_gqa_decode_sel_dev(const uint16_t *k, const uint16_t *v, int64_t n_rows, int n_kv_heads,
+                                 int head_dim, const int32_t *sel, int64_t n_list,
+                                 const uint16_t *q, int n_heads, float scale, float *out,
+                                 void *stream);
+
 /* Replaces the closing of an indexer pool (indexer_absorb, src/attention.c:
  * 486-525; the two projections in front of it, :481-482, stay the caller's
  * GEMVs).  For each of n closed pools: layer-norm statistics of each of the

@@ -1018,3 +1018,48 @@ def test_snapshot_reads_dequantised_rows_and_restores_them(hip, orc):
     rc = hip.lib().cwick_hip_latent_read_f32(lat.h, 1, 1000, 100, f.ctypes.data)
     assert rc == 0 and "capacity" in hip.last_error()
     lat.free(); lat2.free(); ik.free(); ik2.free()
+
+
+# ------------------------------------------------------------------ block-sparse GQA decode
+@pytest.mark.parametrize("n_rows,nh,nkv,hd,bs,keep", [(4096, 16, 4, 256, 64, 8), (700, 8, 8, 128, 16, 5), (3000, 64, 8, 128, 128, 4),
+                                                      (64, 16, 4, 256, 64, 1)])
+def test_gqa_decode_over_selected_blocks(hip, orc, n_rows, nh, nkv, hd, bs, keep):
+    """The attention of the block-sparse decode (src/mm_model.c:1962-2047) over positions expanded
+    from selected blocks as the reference expands them (:1966-1973: whole blocks in the order of
+    selection, clipped to the positions written).  Checked against the oracle's decode over the
+    gathered rows (the same softmax and sums over the same set)."""
+    import torch
+    say("[case] gqa_decode_sel", n_rows, nh, nkv, hd, bs, keep)
+    g = synth.rng(9000 + n_rows)
+    c = synth.cfg2_gqa_prefill(n_rows, nh, nkv, hd, 0, seed=900 + n_rows)
+    cache = hip.KVCache(n_rows, nkv, hd)
+    cache.write(0, c["k"].reshape(n_rows, -1), c["v"].reshape(n_rows, -1))
+    nblk = -(-n_rows // bs)
+    blocks = g.permutation(nblk)[:keep]
+    if nblk - 1 not in blocks:
+        blocks[-1] = nblk - 1                                # the newest block, always (:1752-1757)
+    sel = np.concatenate([np.arange(b * bs, min((b + 1) * bs, n_rows)) for b in blocks]).astype(np.int32)
+    q = c["q"][n_rows - 1]
+    got = hip.gqa_decode_sel(cache, sel, q, c["scale"])
+    ref = orc.gqa_decode(q, c["k"][sel], c["v"][sel], c["scale"])
+    assert_close(got, ref, "gqa_decode_sel %d rows, %d positions" % (n_rows, sel.size))
+    # entries that name no row carry no weight; the order of the list does not matter
+    padded = np.concatenate([[-1, n_rows, -7], sel[::-1], [2 ** 31 - 1]]).astype(np.int32)
+    got2 = hip.gqa_decode_sel(cache, padded, q, c["scale"])
+    assert_close(got2, ref, "gqa_decode_sel padded and reversed")
+    # the whole cache as a list equals the dense decode
+    full = hip.gqa_decode_sel(cache, np.arange(n_rows, dtype=np.int32), q, c["scale"])
+    dense = hip.gqa_decode(cache, n_rows, q, c["scale"])
+    assert np.abs(full - dense).max() <= 1e-6
+    # device operands
+    d_sel = torch.from_numpy(sel).cuda()
+    d_q = torch.from_numpy(q.view(np.int16)).cuda()
+    d_out = torch.empty((nh, hd), dtype=torch.float32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.gqa_decode_sel_dev(cache.k_dev(), cache.v_dev(), n_rows, nkv, hd, d_sel, sel.size, d_q, nh, c["scale"], d_out, s)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_out.cpu().numpy().view(np.uint32), got.view(np.uint32))
+    # nothing valid: zeros
+    none = hip.gqa_decode_sel(cache, np.array([-1, -1, n_rows], np.int32), q, c["scale"])
+    assert np.all(none == 0.0)
+    cache.free()
