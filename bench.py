@@ -424,8 +424,10 @@ def main():
         r3["cpu_baseline"] = cpu
         log("[cpu ] %.0f us/token on %d threads" % (cpu["value"], cpu["cores"]))
     del c3
-    side = {1: (bench_cfg1, a.steps), 2: (bench_cfg2, max(20, a.steps // 10)),
-            4: (bench_cfg4, max(2, a.steps // 100)), 5: (bench_cfg5, max(3, a.steps // 10))}
+    # enough steps that the fixed cost of the two device syncs around the timed region (0.1 to 1 ms
+    # on this stack, whatever is enqueued) stays below a per cent of the region
+    side = {1: (bench_cfg1, a.steps), 2: (bench_cfg2, max(20, a.steps // 4)),
+            4: (bench_cfg4, max(2, a.steps // 50)), 5: (bench_cfg5, max(3, a.steps // 2))}
     for i in sorted(wanted - {3}):
         fn, k = side[i]
         Ti = Timer(hip, torch, k, max(1, min(a.warmup, k // 2)))
