@@ -363,7 +363,6 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                         const f32x4 acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qrope, z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc1);
                         S[kb] += acc * scb;
                     }
-                    S[kb] *= c0;
                 }
                 // positions past the query's last key (only in its last tile)
                 if (t + 1 == tail_tile && tail_keys < TK) {
@@ -376,6 +375,7 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 float lmax = vmax3(S[0][0], S[0][1], vmax(S[0][2], S[0][3]));
 #pragma unroll
                 for (int kb = 1; kb < 4; kb++) lmax = vmax3(lmax, S[kb][0], vmax3(S[kb][1], S[kb][2], S[kb][3]));
+                lmax *= c0;                                   // S stays unscaled: c0 > 0 goes into the exponent's multiply-add
                 const bool moves = __any(lmax > mr + LAZY);   // rare after the first tiles: only then the lanes of a head confer
                 if (moves) {
                     lmax = fmaxf(lmax, __shfl_xor(lmax, 16, 64));
@@ -392,7 +392,7 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 for (int kb = 0; kb < 4; kb++) {
                     f32x4 P;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) P[i] = __builtin_amdgcn_exp2f(S[kb][i] - m_use);
+                    for (int i = 0; i < 4; i++) P[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kb][i], c0, -m_use));
                     lsum += (P[0] + P[1]) + (P[2] + P[3]);
                     u32x2 d;
                     d[0] = pack_f16_rne(P[0], P[1]);
