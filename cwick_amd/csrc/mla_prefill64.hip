@@ -157,8 +157,15 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
 
     const int n_hb = (p.nh + HW - 1) / HW;
     const int64_t total = (int64_t)gridDim.x;
+    // Workgroups go to the eight XCDs round robin.  The head blocks of a query run on one XCD (they
+    // read the same tiles at the same time: one fetch into that L2), and consecutive queries go
+    // to consecutive XCDs, so that every XCD gets the same mix of long and short queries (a
+    // contiguous eighth of the queries per XCD left the XCD with the longest ones 6 % behind).
     int64_t unit = blockIdx.x;
-    if (total % 8 == 0) unit = (unit % 8) * (total / 8) + unit / 8;   // neighbours in the order of work share an XCD
+    if (total % (8 * n_hb) == 0) {
+        const int64_t grp = unit / (8 * n_hb), r = unit % (8 * n_hb);
+        unit = (8 * grp + r % 8) * n_hb + r / 8;
+    }
     const int hb = (int)(unit % n_hb);
     const int y = p.nq - 1 - (int)(unit / n_hb);                      // the queries with the most keys start first
 
