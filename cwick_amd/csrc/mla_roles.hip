@@ -211,8 +211,19 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 
     const int n_hb = (p.nh + HW - 1) / HW;
     const int64_t total = (int64_t)gridDim.x;
+    // Workgroups go to the eight XCDs round robin.  Decode: an XCD takes a contiguous eighth of
+    // the units (the head blocks of a slice, the slices of a query: what they share stays in one
+    // L2).  Causal prefill: queries differ in length, so consecutive queries go to consecutive
+    // XCDs instead (a contiguous eighth would leave the XCD with the longest queries behind).
     int64_t unit = blockIdx.x;
-    if (total % 8 == 0) unit = (unit % 8) * (total / 8) + unit / 8;
+    if (p.list_step > 0 && p.n_splits == 1) {
+        if (total % (8 * n_hb) == 0) {
+            const int64_t grp = unit / (8 * n_hb), r = unit % (8 * n_hb);
+            unit = (8 * grp + r % 8) * n_hb + r / 8;
+        }
+    } else if (total % 8 == 0) {
+        unit = (unit % 8) * (total / 8) + unit / 8;
+    }
     const int hb = (int)(unit % n_hb);
     const int split = (int)((unit / n_hb) % p.n_splits);
     int y = (int)(unit / ((int64_t)n_hb * p.n_splits));
