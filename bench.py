@@ -465,6 +465,8 @@ def main():
         "checked": all(r.get("checked", False) for r in results.values()) if orc else None,
         "measured_ceilings": {k: round(v, 1) for k, v in CEIL.items()} or None,
         "roofline": r3["roofline"],
+        "traffic_source": "profiles/hot_kernels_pmc_traffic.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE of the same "
+                          "command, scaled by a 256 MiB copy; not measured in this run)",
         "roofline_mfma": r3["roofline_mfma"],
         "cpu_baseline": cpu,
         "configs": results,
