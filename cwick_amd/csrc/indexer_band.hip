@@ -42,6 +42,14 @@ constexpr int IB_KEYS = CWICK_INDEXER_APPROX_KEYS;   // keys per workgroup of th
 constexpr int IB_HD = CWICK_HIP_INDEX_DIM;    // 128
 
 typedef __attribute__((ext_vector_type(2))) float ib_f32x2;
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+
+// v[l] + v[l ^ 32] in every lane: the two halves of the wave trade places between two copies
+__device__ __forceinline__ float ib_half_sum(float v) {
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a + b;
+}
 
 __global__ void __launch_bounds__(IB_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict__ kscale,
@@ -51,7 +59,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
                       IndexerBandRow *__restrict__ rows,
                       uint32_t *__restrict__ digit0, size_t digit0_row) {   // optional: first-digit counts for the radix select
-    __shared__ float c_sh[2][IB_HD];
+    __shared__ __attribute__((aligned(16))) float cpart_sh[16][IB_HD];
+    __shared__ __attribute__((aligned(16))) uint16_t cb_sh[IB_HD + 64];          // coefficients, then 128 bytes of zeros
     __shared__ uint32_t hist0[256 * 8];
     __shared__ __attribute__((aligned(16))) uint16_t q_sh[64 * IB_QROW];
     __shared__ float w_sh[64];
@@ -73,8 +82,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     const int64_t wbase = (int64_t)wg * IB_KEYS + (int64_t)wave * (IB_KEYS / 4);
     constexpr int N_IT = IB_KEYS / 4 / 32;
     // the key bytes and the scale of an iteration are loaded two iterations ahead
-    u32x4 raw_a[4], raw_b[4];
-    float kst_a, kst_b;
+    u32x4 raw_a[4], raw_b[4], raw_c[4];
+    float kst_a, kst_b, kst_c;
     auto load_keys = [&](int it, u32x4 (&raw)[4], float &kst) {
         int64_t tc = wbase + (it < N_IT ? it : N_IT - 1) * 32 + row;
         tc = tc < n_keys ? tc : n_keys - 1;
@@ -87,9 +96,20 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     // (sixteen bytes per thread and step) and the waves take their fragments from LDS; rows are
     // 272 bytes apart there, which spreads the sixteen-byte reads of consecutive heads over the
     // banks.  The loads go out first and the first two key iterations right behind them.
-    bf16x8 qa[2][8], ca[8];
+    // c_i = sum_h |w_h| |q_hi| starts from the same registers: thread (group = tid / 16, part =
+    // tid % 16) holds dims 8 part .. +7 of heads group + 16 j, adds up its four heads and leaves
+    // the eight sums in LDS; after the barrier thread i < 128 adds the sixteen groups of dim i.
+    bf16x8 qa[2][8];
     {
+        // (the weights first: a load that is waited for drags every load issued before it along)
+        const float w_mine = (tid < 64 && tid < ih) ? wb[tid] : 0.0f;
+        float w4[4];
         u32x4 stage[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int head = (tid >> 4) + 16 * j;
+            w4[j] = head < ih ? fabsf(wb[head]) : 0.0f;
+        }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int c = tid + IB_THREADS * j, head = c >> 4, part = c & 15;
@@ -99,13 +119,22 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         }
         load_keys(0, raw_a, kst_a);
         load_keys(1, raw_b, kst_b);
+        float cp[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int c = tid + IB_THREADS * j;
             *(u32x4 *)&q_sh[(c >> 4) * IB_QROW + 8 * (c & 15)] = stage[j];
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t x = stage[j][d];
+                cp[2 * d] = __builtin_fmaf(w4[j], __builtin_bit_cast(float, (x << 16) & 0x7FFFFFFFu), cp[2 * d]);
+                cp[2 * d + 1] = __builtin_fmaf(w4[j], __builtin_bit_cast(float, x & 0x7FFF0000u), cp[2 * d + 1]);
+            }
         }
+        *(f32x4 *)&cpart_sh[tid >> 4][8 * (tid & 15)] = (f32x4){cp[0], cp[1], cp[2], cp[3]};
+        *(f32x4 *)&cpart_sh[tid >> 4][8 * (tid & 15) + 4] = (f32x4){cp[4], cp[5], cp[6], cp[7]};
+        if (tid < 64) w_sh[tid] = w_mine;
     }
-    if (tid < 64) w_sh[tid] = tid < ih ? wb[tid] : 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) hist0[tid + IB_THREADS * j] = 0u;
     __syncthreads();
@@ -114,32 +143,20 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
 #pragma unroll
         for (int ks = 0; ks < 8; ks++)
             qa[mb][ks] = *(const bf16x8 *)&q_sh[(mb * 32 + row) * IB_QROW + 64 * g + 8 * ks];
-    {   // c_i = sum_h |w_h| |q_hi|: thread (i, half) adds up 32 heads of dimension i out of LDS
-        const int i = tid & (IB_HD - 1), half = tid >> 7;
-        float c = 0.0f;
-#pragma unroll 8
-        for (int h = 0; h < 32; h++) {
-            const int head = 32 * half + h;
-            c = __builtin_fmaf(fabsf(w_sh[head]), fabsf(bf16_to_f32(q_sh[head * IB_QROW + i])), c);
-        }
-        c_sh[half][i] = c;
+    if (tid < IB_HD) {
+        float part[16], c = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) part[k] = cpart_sh[k][tid];
+#pragma unroll
+        for (int k = 0; k < 16; k++) c += part[k];
+        cb_sh[tid] = (uint16_t)((__builtin_bit_cast(uint32_t, c) + 0xFFFFu) >> 16);     // rounded up to bf16
+        if (tid < 64) cb_sh[IB_HD + tid] = 0;
     }
     __syncthreads();
-#pragma unroll
-    for (int ks = 0; ks < 8; ks++) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (row == 0) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                // rounded up to bf16
-                const int i0 = 64 * g + 8 * ks + 2 * j;
-                const uint32_t lo = (__builtin_bit_cast(uint32_t, c_sh[0][i0] + c_sh[1][i0]) + 0xFFFFu) >> 16;
-                const uint32_t hi = (__builtin_bit_cast(uint32_t, c_sh[0][i0 + 1] + c_sh[1][i0 + 1]) + 0xFFFFu) >> 16;
-                v[j] = lo | (hi << 16);
-            }
-        }
-        ca[ks] = __builtin_bit_cast(bf16x8, v);
-    }
+    // the bound row's A fragments are read from LDS step by step: lanes of row 0 from the
+    // coefficients, all others from a stretch of zeros behind them
+    const char __attribute__((address_space(3))) *c_lane =
+        (const char __attribute__((address_space(3))) *)&cb_sh[row == 0 ? 64 * g : IB_HD];
     // the heads this lane holds after the MFMAs: register i of block mb is head
     // 32 mb + 8 (i / 4) + 4 g + i % 4
     float wl[2][16];
@@ -152,41 +169,60 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     auto iteration = [&](int it, const u32x4 (&raw)[4], float kst) {
         const int64_t t = wbase + it * 32 + row;
         const bool live = t < n_keys;
-        // the accumulators are pinned to VGPRs (through the builtin they land in AGPRs and cost a
-        // read each); the compiler does not see these as MFMAs and leaves out the wait states
-        // they need: two between a VALU write of an operand and the MFMA that reads it (the
-        // s_nop 1 in front of the first MFMA after the conversions and of the one after the
-        // masks), and the wait before the results are read
+        // The accumulators are pinned to VGPRs (through the builtin they land in AGPRs and cost a
+        // read each).  The compiler does not see these as MFMAs and leaves out the wait states
+        // they need (one state = four cycles = one pass of the matrix pipe): two between a VALU
+        // write of an operand and the MFMA that reads it, up to nineteen between the issue of
+        // an MFMA and a VALU read of its result.  The first is met by converting the keys
+        // of k-step ks + 1 before the MFMAs of k-step ks are issued (which also puts the
+        // conversions in the shadow of the matrix pipe), the second by the s_nop behind the loop.
         f32x16 d0, d1, ab;
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            typedef __attribute__((ext_vector_type(2))) __bf16 ib_bf16x2;
-            u32x4 e;
+        typedef __attribute__((ext_vector_type(2))) __bf16 ib_bf16x2;
+        u32x4 e[2], ea[2], cfrag[2];
+        auto convert = [&](int ks, u32x4 &eo, u32x4 &eao) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {                          // exact: E4M3 fits bf16
                 const int dw = raw[ks >> 1][2 * (ks & 1) + j];
-                e[2 * j] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, false));
-                e[2 * j + 1] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, true));
+                eo[2 * j] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, false));
+                eo[2 * j + 1] = __builtin_bit_cast(uint32_t, (ib_bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(dw, 1.0f, true));
             }
-            u32x4 ea;
 #pragma unroll
-            for (int j = 0; j < 4; j++) ea[j] = e[j] & 0x7FFF7FFFu;
+            for (int j = 0; j < 4; j++) eao[j] = eo[j] & 0x7FFF7FFFu;
+        };
+        convert(0, e[0], ea[0]);
+        cfrag[0] = *(const lds_u32x4 *)(c_lane);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            const u32x4 ea_before = ea[nxt], c_before = cfrag[nxt];   // operands of the last MFMA issued
+            if (ks + 1 < 8) {
+                convert(ks + 1, e[nxt], ea[nxt]);
+                cfrag[nxt] = *(const lds_u32x4 *)(c_lane + 16 * (ks + 1));
+            }
+            // Everything above is in its registers before the first MFMA below is issued; the
+            // operands of the step before stay allocated up to here (an MFMA goes on reading its
+            // operands for a while after it has been issued, and the compiler, which does not
+            // know, would hand their registers to the conversions above).
+            if (ks == 0)
+                asm volatile("s_nop 1" : "+v"(e[nxt]), "+v"(ea[nxt]), "+v"(e[cur]), "+v"(ea[cur]), "+v"(cfrag[cur]));
+            else
+                asm volatile("" : "+v"(e[nxt]), "+v"(ea[nxt]), "+v"(e[cur]), "+v"(ea[cur]), "+v"(cfrag[cur])
+                             : "v"(ea_before), "v"(c_before));
             if (ks == 0) {
-                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d0) : "v"(qa[0][ks]), "v"(e));
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d1) : "v"(qa[1][ks]), "v"(e));
-                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(ab) : "v"(ca[ks]), "v"(ea));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d0) : "v"(qa[0][ks]), "v"(e[cur]));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d1) : "v"(qa[1][ks]), "v"(e[cur]));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(ab) : "v"(cfrag[cur]), "v"(ea[cur]), "v"(e[cur]));
             } else {
-                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d0) : "v"(qa[0][ks]), "v"(e));
-                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d1) : "v"(qa[1][ks]), "v"(e));
-                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ab) : "v"(ca[ks]), "v"(ea));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d0) : "v"(qa[0][ks]), "v"(e[cur]));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d1) : "v"(qa[1][ks]), "v"(e[cur]));
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ab) : "v"(cfrag[cur]), "v"(ea[cur]), "v"(e[cur]));
             }
         }
-        // Nothing may write a register that these MFMAs read before they are done (they read
-        // their operands pass by pass, and the compiler does not know them as MFMAs): the
-        // instructions that follow the last one wait, and carry the accumulators, so that
-        // nothing that reads those can be scheduled above the wait either.
-        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d0), "+v"(d1), "+v"(ab)::"memory");
-        float sp = 0.0f;
+        // Nothing may read the results or write a register that these MFMAs read before the last
+        // one is through: the wait carries the accumulators, so that nothing that reads them can
+        // be scheduled above it either.
+        asm volatile("s_nop 15\n\ts_nop 2" : "+v"(d0), "+v"(d1), "+v"(ab)::"memory");
+        float sp = 0.0f, sq = 0.0f, sr = 0.0f, ss = 0.0f;      // four chains: a dependent FMA waits for the one before it
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             // one instruction per ReLU (through fmaxf or fmed3 the compiler adds a second one
@@ -194,11 +230,18 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
             float r0, r1;
             asm("v_max_f32 %0, 0, %1" : "=v"(r0) : "v"(d0[i]));
             asm("v_max_f32 %0, 0, %1" : "=v"(r1) : "v"(d1[i]));
-            sp = __builtin_fmaf(wl[0][i], r0, sp);
-            sp = __builtin_fmaf(wl[1][i], r1, sp);
+            if (i & 1) {
+                sr = __builtin_fmaf(wl[0][i], r0, sr);
+                ss = __builtin_fmaf(wl[1][i], r1, ss);
+            } else {
+                sp = __builtin_fmaf(wl[0][i], r0, sp);
+                sq = __builtin_fmaf(wl[1][i], r1, sq);
+            }
         }
-        sp += __shfl_xor(sp, 32, 64);
-        const float band = ab[0] + __shfl_xor(ab[0], 32, 64);      // row 0 sits in the g = 0 lanes
+        sp = (sp + sq) + (sr + ss);
+        // lane l + lane l ^ 32 without a trip through LDS
+        sp = ib_half_sum(sp);
+        const float band = ib_half_sum(ab[0]);                     // row 0 sits in the g = 0 lanes
         const float st = sp * kst;
         const float beta = band * fabsf(kst) * (512.0f / 16777216.0f);
         if (live && g == 0) {
@@ -209,21 +252,20 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         }
         if (live) bmax = (beta <= bmax) ? bmax : beta;             // NaN sticks
     };
-#pragma unroll 1
-    for (int it = 0; it < N_IT; it += 2) {
+    // three register sets in turn, so that the loads of iteration it + 2 go out before
+    // iteration it computes and nothing is copied between sets (a copy waits for its load);
+    // unrolled, so that every wait counts exactly the loads behind the one it needs
+#pragma unroll
+    for (int it = 0; it < N_IT; it += 3) {
         if (wbase + it * 32 >= n_keys) break;                      // wave-uniform
-        u32x4 raw[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) raw[i] = raw_a[i];
-        float kst = kst_a;
-        load_keys(it + 2, raw_a, kst_a);
-        iteration(it, raw, kst);
-        if (wbase + (it + 1) * 32 >= n_keys) break;
-#pragma unroll
-        for (int i = 0; i < 4; i++) raw[i] = raw_b[i];
-        kst = kst_b;
-        load_keys(it + 3, raw_b, kst_b);
-        iteration(it + 1, raw, kst);
+        load_keys(it + 2, raw_c, kst_c);
+        iteration(it, raw_a, kst_a);
+        if (it + 1 >= N_IT || wbase + (it + 1) * 32 >= n_keys) break;
+        load_keys(it + 3, raw_a, kst_a);
+        iteration(it + 1, raw_b, kst_b);
+        if (it + 2 >= N_IT || wbase + (it + 2) * 32 >= n_keys) break;
+        load_keys(it + 4, raw_b, kst_b);
+        iteration(it + 2, raw_c, kst_c);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
