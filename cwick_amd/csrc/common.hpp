@@ -70,7 +70,7 @@ struct IndexerBandRow {
     uint32_t fallback;    // the band could not be formed (bound not finite, NaN threshold)
 };
 constexpr int CWICK_INDEXER_BAND_CAP = 4096;   // candidate list entries per row
-constexpr int CWICK_INDEXER_APPROX_KEYS = 1024;   // keys per workgroup (= per bound slot) of the approximate kernel
+constexpr int CWICK_INDEXER_APPROX_KEYS = 2048;   // keys per workgroup (= per bound slot) of the approximate kernel
 inline int indexer_approx_slots(int64_t n_keys) {
     return (int)((n_keys + CWICK_INDEXER_APPROX_KEYS - 1) / CWICK_INDEXER_APPROX_KEYS);
 }

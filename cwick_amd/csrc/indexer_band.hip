@@ -36,7 +36,8 @@
 
 namespace cwick {
 
-constexpr int IB_THREADS = 256;
+constexpr int IB_THREADS = 512;
+constexpr int IB_WAVES = IB_THREADS / 64;
 constexpr int IB_QROW = 128 + 8;                 // bf16 per head row of q in LDS (padded: 272 bytes)
 constexpr int IB_KEYS = CWICK_INDEXER_APPROX_KEYS;   // keys per workgroup of the approximate kernel
 constexpr int IB_HD = CWICK_HIP_INDEX_DIM;    // 128
@@ -59,7 +60,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
                       int ih, float *__restrict__ scores, float *__restrict__ beta_slots,
                       IndexerBandRow *__restrict__ rows,
                       uint32_t *__restrict__ digit0, size_t digit0_row) {   // optional: first-digit counts for the radix select
-    __shared__ __attribute__((aligned(16))) float cpart_sh[16][IB_HD];
+    __shared__ __attribute__((aligned(16))) float cpart_sh[IB_THREADS / 16][IB_HD];
     __shared__ __attribute__((aligned(16))) uint16_t cb_sh[IB_HD + 64];          // coefficients, then 128 bytes of zeros
     __shared__ uint32_t hist0[256 * 8];
     __shared__ __attribute__((aligned(16))) uint16_t q_sh[64 * IB_QROW];
@@ -79,8 +80,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     const int row = lane & 31, g = lane >> 5;
     const uint8_t *kb = keys + (size_t)b * key_bstride;
     const float *ksb = kscale + (size_t)b * kscale_bstride;
-    const int64_t wbase = (int64_t)wg * IB_KEYS + (int64_t)wave * (IB_KEYS / 4);
-    constexpr int N_IT = IB_KEYS / 4 / 32;
+    const int64_t wbase = (int64_t)wg * IB_KEYS + (int64_t)wave * (IB_KEYS / IB_WAVES);
+    constexpr int N_IT = IB_KEYS / IB_WAVES / 32;
     // the key bytes and the scale of an iteration are loaded two iterations ahead
     u32x4 raw_a[4], raw_b[4], raw_c[4];
     float kst_a, kst_b, kst_c;
@@ -103,15 +104,16 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
     {
         // (the weights first: a load that is waited for drags every load issued before it along)
         const float w_mine = (tid < 64 && tid < ih) ? wb[tid] : 0.0f;
-        float w4[4];
-        u32x4 stage[4];
+        constexpr int NST = 1024 / IB_THREADS;              // sixteen-byte pieces of q per thread
+        float w4[NST];
+        u32x4 stage[NST];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int head = (tid >> 4) + 16 * j;
+        for (int j = 0; j < NST; j++) {
+            const int head = (tid >> 4) + (IB_THREADS / 16) * j;
             w4[j] = head < ih ? fabsf(wb[head]) : 0.0f;
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NST; j++) {
             const int c = tid + IB_THREADS * j, head = c >> 4, part = c & 15;
             const int hc = head < ih ? head : ih - 1;           // clamped load, zeroed afterwards
             stage[j] = *(const u32x4 *)(qb + (size_t)hc * IB_HD + 8 * part);
@@ -121,7 +123,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         load_keys(1, raw_b, kst_b);
         float cp[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NST; j++) {
             const int c = tid + IB_THREADS * j;
             *(u32x4 *)&q_sh[(c >> 4) * IB_QROW + 8 * (c & 15)] = stage[j];
 #pragma unroll
@@ -136,7 +138,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         if (tid < 64) w_sh[tid] = w_mine;
     }
 #pragma unroll
-    for (int j = 0; j < 8; j++) hist0[tid + IB_THREADS * j] = 0u;
+    for (int j = 0; j < 2048 / IB_THREADS; j++) hist0[tid + IB_THREADS * j] = 0u;
     __syncthreads();
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
@@ -144,11 +146,11 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         for (int ks = 0; ks < 8; ks++)
             qa[mb][ks] = *(const bf16x8 *)&q_sh[(mb * 32 + row) * IB_QROW + 64 * g + 8 * ks];
     if (tid < IB_HD) {
-        float part[16], c = 0.0f;
+        float part[IB_THREADS / 16], c = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 16; k++) part[k] = cpart_sh[k][tid];
+        for (int k = 0; k < IB_THREADS / 16; k++) part[k] = cpart_sh[k][tid];
 #pragma unroll
-        for (int k = 0; k < 16; k++) c += part[k];
+        for (int k = 0; k < IB_THREADS / 16; k++) c += part[k];
         cb_sh[tid] = (uint16_t)((__builtin_bit_cast(uint32_t, c) + 0xFFFFu) >> 16);     // rounded up to bf16
         if (tid < 64) cb_sh[IB_HD + tid] = 0;
     }
@@ -280,7 +282,7 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         for (int i = 1; i < IB_THREADS / 64; i++) m = (bmax_sh[i] <= m) ? m : bmax_sh[i];
         beta_slots[(size_t)b * gridDim.x + wg] = m;
     }
-    if (digit0) {
+    if (digit0 && tid < 256) {
         uint32_t c = 0u;
 #pragma unroll
         for (int j = 0; j < 8; j++) c += hist0[tid * 8 + ((j + tid) & 7)];
@@ -391,7 +393,7 @@ int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_
                           const float *w, int n_idx_heads, float *scores, float *beta_slots,
                           IndexerBandRow *rows, uint32_t *digit0_slices, size_t digit0_row_dwords,
                           hipStream_t s) {
-    static_assert(IB_THREADS == 256, "one thread per first-digit bin");
+    static_assert(IB_THREADS >= 256 && 1024 % IB_THREADS == 0, "a thread per first-digit bin, whole pieces of q per thread");
     CWICK_REQUIRE(keys && kscale && q_idx && w && scores && beta_slots && rows, "indexer_approx: null pointer");
     CWICK_REQUIRE(n_keys >= 1 && n_idx_heads >= 1 && n_idx_heads <= 64, "indexer_approx: shape out of range");
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,

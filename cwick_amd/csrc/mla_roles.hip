@@ -85,7 +85,18 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 // the larger of two values; a NaN on either side wins
-__device__ __forceinline__ float nan_max(float a, float b) { return (a != a || a > b) ? a : b; }
+// max(v[l], v[l ^ 16]) and max(v[l], v[l ^ 32]) in every lane: rows of sixteen lanes (halves of
+// the wave) trade places between two copies of the value
+__device__ __forceinline__ uint32_t lanes_xor16_max(uint32_t v) {
+    uint32_t a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a > b ? a : b;
+}
+__device__ __forceinline__ uint32_t lanes_xor32_max(uint32_t v) {
+    uint32_t a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a > b ? a : b;
+}
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -210,23 +221,24 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
     const int g = lane >> 4;         // 32-wide contraction block (QK) / 8-wide (PV)
 
     const int n_hb = (p.nh + HW - 1) / HW;
-    const int64_t total = (int64_t)gridDim.x;
+    const uint32_t total = gridDim.x, u_hb = (uint32_t)n_hb, u_sp = (uint32_t)p.n_splits;
     // Workgroups go to the eight XCDs round robin.  Decode: an XCD takes a contiguous eighth of
     // the units (the head blocks of a slice, the slices of a query: what they share stays in one
     // L2).  Causal prefill: queries differ in length, so consecutive queries go to consecutive
     // XCDs instead (a contiguous eighth would leave the XCD with the longest queries behind).
-    int64_t unit = blockIdx.x;
+    // (32-bit arithmetic: a 64-bit division is a hundred instructions in front of the first load)
+    uint32_t unit = blockIdx.x;
     if (p.list_step > 0 && p.n_splits == 1) {
-        if (total % (8 * n_hb) == 0) {
-            const int64_t grp = unit / (8 * n_hb), r = unit % (8 * n_hb);
-            unit = (8 * grp + r % 8) * n_hb + r / 8;
+        if (total % (8 * u_hb) == 0) {
+            const uint32_t grp = unit / (8 * u_hb), r = unit % (8 * u_hb);
+            unit = (8 * grp + r % 8) * u_hb + r / 8;
         }
     } else if (total % 8 == 0) {
         unit = (unit % 8) * (total / 8) + unit / 8;
     }
-    const int hb = (int)(unit % n_hb);
-    const int split = (int)((unit / n_hb) % p.n_splits);
-    int y = (int)(unit / ((int64_t)n_hb * p.n_splits));
+    const int hb = (int)(unit % u_hb);
+    const int split = (int)((unit / u_hb) % u_sp);
+    int y = (int)(unit / (u_hb * u_sp));
     if (p.list_step > 0) y = p.nq - 1 - y;          // causal prefill: the queries with the most keys start first
 
     const uint8_t *rows = p.rows + (size_t)y * p.row_bstride;
@@ -703,14 +715,25 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             // The partial leaves as 16-bit fixed point: this wave's 128 dims of the head share one
             // scale, their largest magnitude, so every value is off by at most 2^-16 of that.  A
             // non-finite value makes the scale NaN and with it the head's merged output.
-            float big = 0.0f;   // in accumulator units
+            // (the largest magnitude as an integer maximum of the bit patterns without their signs:
+            // infinities and NaNs compare above every finite value; four chains, because each link
+            // waits for the one before it, and the four lanes of a head meet without a trip
+            // through LDS)
+            uint32_t b0 = 0u, b1 = 0u, b2 = 0u, b3 = 0u;
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) big = nan_max(big, __builtin_fabsf(oacc[h2][j][i]));
-            big = nan_max(big, __shfl_xor(big, 16));
-            big = nan_max(big, __shfl_xor(big, 32));
-            if (!(big < INFINITY)) big = __builtin_nanf("");
+            for (int j = 0; j < 8; j++) {
+                const u32x4 a = __builtin_bit_cast(u32x4, oacc[h2][j]) & 0x7FFFFFFFu;
+                b0 = a[0] > b0 ? a[0] : b0;
+                b1 = a[1] > b1 ? a[1] : b1;
+                b2 = a[2] > b2 ? a[2] : b2;
+                b3 = a[3] > b3 ? a[3] : b3;
+            }
+            uint32_t bm = b0 > b1 ? b0 : b1;
+            const uint32_t bn = b2 > b3 ? b2 : b3;
+            bm = bm > bn ? bm : bn;
+            bm = lanes_xor16_max(bm);
+            bm = lanes_xor32_max(bm);
+            float big = bm > 0x7F7FFFFFu ? __builtin_nanf("") : __builtin_bit_cast(float, bm);   // in accumulator units
             const float to_unit = big > 0.0f ? 1.0f / big : 0.0f;
             uint32_t *pq = p.part_acc + (pb * NDB + 8 * cw) * 128 + lane * 2;   // [db][lane][4 x i16]
 #pragma unroll
