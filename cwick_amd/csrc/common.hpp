@@ -208,10 +208,46 @@ __device__ __forceinline__ uint32_t e4m3x2_to_bf16x2(uint32_t w) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// Lane l meets lane l ^ 16 (l ^ 32) without a trip through LDS: the rows of sixteen lanes (the
+// halves of the wave) trade places between two copies of the value, and a commutative
+// operation on the two copies is what a butterfly step would give, bit for bit.
+__device__ __forceinline__ void lanes_swap16(uint32_t &a, uint32_t &b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void lanes_swap32(uint32_t &a, uint32_t &b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float xor16_max(float v) {
+    uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+    lanes_swap16(a, b);
+    return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ __forceinline__ float xor32_max(float v) {
+    uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+    lanes_swap32(a, b);
+    return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ __forceinline__ float xor16_sum(float v) {
+    uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+    lanes_swap16(a, b);
+    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+__device__ __forceinline__ float xor32_sum(float v) {
+    uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+    lanes_swap32(a, b);
+    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+// the maximum over the wave in every lane: within a row of sixteen lanes through DPP (swap in
+// pairs, swap pairs, mirror the half row, mirror the row), then the two steps above
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+#define CWICK_DPP_MAX(ctrl)                                                                                   \
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, false)))
+    CWICK_DPP_MAX(0xB1);     // quad_perm [1, 0, 3, 2]
+    CWICK_DPP_MAX(0x4E);     // quad_perm [2, 3, 0, 1]
+    CWICK_DPP_MAX(0x141);    // row_half_mirror
+    CWICK_DPP_MAX(0x140);    // row_mirror
+#undef CWICK_DPP_MAX
+    return xor32_max(xor16_max(v));
 }
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -241,11 +241,12 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 qv[8 * c + 2 * d + 1] = bf16hi_to_f32(w[d]);
             }
         }
-        float amax = 0.0f;
+        float am4[4] = {0.0f, 0.0f, 0.0f, 0.0f};      // four chains: a link waits for the one before it
 #pragma unroll
-        for (int j = 0; j < 32; j++) amax = fmaxf(amax, __builtin_fabsf(qv[j]));
-        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        for (int j = 0; j < 32; j++) am4[j & 3] = fmaxf(am4[j & 3], __builtin_fabsf(qv[j]));
+        float amax = fmaxf(fmaxf(am4[0], am4[1]), fmaxf(am4[2], am4[3]));
+        amax = xor16_max(amax);
+        amax = xor32_max(amax);
         int s = amax > 0.0f ? (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu) - 127 - 7 : 0;
         s = s < -110 ? -110 : s;
         const float inv = pow2i(-s), mul = pow2i(s);
@@ -390,8 +391,8 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 lmax *= c0;                                   // S stays unscaled: c0 > 0 goes into the exponent's multiply-add
                 const bool moves = __any(lmax > mr + LAZY);   // rare after the first tiles: only then the lanes of a head confer
                 if (moves) {
-                    lmax = fmaxf(lmax, __shfl_xor(lmax, 16, 64));
-                    lmax = fmaxf(lmax, __shfl_xor(lmax, 32, 64));
+                    lmax = xor16_max(lmax);
+                    lmax = xor32_max(lmax);
                     const float m_new = lmax > mr + LAZY ? lmax : mr;
                     const float cf = (mr == -INFINITY || m_new == mr) ? 1.0f : __builtin_amdgcn_exp2f(mr - m_new);
                     l_priv *= cf;
@@ -421,8 +422,8 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
 
         // ---- the sums of the scoring role meet in LDS (the exchange area is free now) ----
         float *lsum = reinterpret_cast<float *>(&sm.x[0]);            // [16-head block][head]
-        float ls = l_priv + __shfl_xor(l_priv, 16, 64);
-        ls += __shfl_xor(ls, 32, 64);
+        float ls = xor16_sum(l_priv);
+        ls = xor32_sum(ls);
         if (g == 0) lsum[hq * 16 + n] = ls;
         LDS_BARRIER();
     } else {
@@ -475,8 +476,7 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                     smax = smax > sb[15] ? smax : sb[15];
                     if (__any(smax >= thr_bits && smax != 0u)) {
                         float sm_f = __builtin_bit_cast(float, smax);
-#pragma unroll
-                        for (int o = 32; o > 0; o >>= 1) sm_f = fmaxf(sm_f, __shfl_xor(sm_f, o, 64));
+                        sm_f = wave_max(sm_f);
                         const int e_tile = (int)((__builtin_bit_cast(uint32_t, sm_f) >> 23) & 0xFFu) - 126;
                         if (e_tile > e_run) {
                             if (e_run != E_NONE) ecorr = pow2i(e_run - e_tile);

@@ -84,17 +84,15 @@ constexpr int MERGE_MAX_SPLITS = 1024;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-// the larger of two values; a NaN on either side wins
-// max(v[l], v[l ^ 16]) and max(v[l], v[l ^ 32]) in every lane: rows of sixteen lanes (halves of
-// the wave) trade places between two copies of the value
+// max(v[l], v[l ^ 16]) and max(v[l], v[l ^ 32]) in every lane
 __device__ __forceinline__ uint32_t lanes_xor16_max(uint32_t v) {
     uint32_t a = v, b = v;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    lanes_swap16(a, b);
     return a > b ? a : b;
 }
 __device__ __forceinline__ uint32_t lanes_xor32_max(uint32_t v) {
     uint32_t a = v, b = v;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    lanes_swap32(a, b);
     return a > b ? a : b;
 }
 typedef __attribute__((ext_vector_type(8))) int i32x8;
@@ -344,11 +342,12 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                     qv[8 * c + 2 * d + 1] = bf16hi_to_f32(w[d]);
                 }
             }
-            float amax = 0.0f;
+            float am4[4] = {0.0f, 0.0f, 0.0f, 0.0f};      // four chains: a link waits for the one before it
 #pragma unroll
-            for (int j = 0; j < 32; j++) amax = fmaxf(amax, __builtin_fabsf(qv[j]));
-            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            for (int j = 0; j < 32; j++) am4[j & 3] = fmaxf(am4[j & 3], __builtin_fabsf(qv[j]));
+            float amax = fmaxf(fmaxf(am4[0], am4[1]), fmaxf(am4[2], am4[3]));
+            amax = xor16_max(amax);
+            amax = xor32_max(amax);
             int s = amax > 0.0f ? (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu) - 127 - 7 : 0;
             s = s < -110 ? -110 : s;
             const float inv = pow2i(-s), mul = pow2i(s);
@@ -509,8 +508,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 float m_loc = mr;
                 const bool moves = __any(lmax > mr + LAZY);   // rare after the first tiles: only then the lanes of a head confer
                 if (moves) {
-                    lmax = fmaxf(lmax, __shfl_xor(lmax, 16, 64));
-                    lmax = fmaxf(lmax, __shfl_xor(lmax, 32, 64));
+                    lmax = xor16_max(lmax);
+                    lmax = xor32_max(lmax);
                     m_loc = lmax > mr + LAZY ? lmax : mr;
                 }
                 const float m_use = m_loc == -INFINITY ? 0.0f : m_loc;
@@ -538,8 +537,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
 
         // ---- the sums of the scoring role meet in LDS (the exchange area is free now) ----
         float *lsum = reinterpret_cast<float *>(&sm.x[0]);            // [head half][head][key block]
-        float ls = l_priv + __shfl_xor(l_priv, 16, 64);
-        ls += __shfl_xor(ls, 32, 64);
+        float ls = xor16_sum(l_priv);
+        ls = xor32_sum(ls);
         if (g == 0) lsum[(hh * 16 + n) * 4 + kb] = ls;
         LDS_BARRIER();
     } else {
@@ -605,8 +604,7 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                     smax = smax > sb[15] ? smax : sb[15];
                     if (__any(smax >= thr_bits && smax != 0u)) {
                         float sm_f = __builtin_bit_cast(float, smax);
-#pragma unroll
-                        for (int o = 32; o > 0; o >>= 1) sm_f = fmaxf(sm_f, __shfl_xor(sm_f, o, 64));
+                        sm_f = wave_max(sm_f);
                         const int e_tile = (int)((__builtin_bit_cast(uint32_t, sm_f) >> 23) & 0xFFu) - 126;
                         if (e_tile > e_run) {
                             if (e_run != E_NONE) ecorr = pow2i(e_run - e_tile);
