@@ -237,8 +237,52 @@ __device__ __forceinline__ float xor32_sum(float v) {
     lanes_swap32(a, b);
     return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
 }
-// the maximum over the wave in every lane: within a row of sixteen lanes through DPP (swap in
-// pairs, swap pairs, mirror the half row, mirror the row), then the two steps above
+// Reductions and scans over the wave without LDS.  Within a row of sixteen lanes through DPP:
+// swap in pairs, swap pairs, mirror the half row, mirror the row (every step joins two groups
+// of lanes that already agree, so all lanes end with the result); across rows the two swaps
+// above.  A scan shifts within the row by 1, 2, 4, 8 and then hands the last lane of a row to
+// the rows behind it.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xF, false);   // lanes without a source read 0
+}
+#define CWICK_WAVE_ALLREDUCE(v, OP)                                                         \
+    do {                                                                                    \
+        { const uint32_t o_ = dpp_u32<0xB1, 0xF>(v); v = OP(v, o_); }   /* quad_perm [1,0,3,2] */ \
+        { const uint32_t o_ = dpp_u32<0x4E, 0xF>(v); v = OP(v, o_); }   /* quad_perm [2,3,0,1] */ \
+        { const uint32_t o_ = dpp_u32<0x141, 0xF>(v); v = OP(v, o_); }  /* row_half_mirror */      \
+        { const uint32_t o_ = dpp_u32<0x140, 0xF>(v); v = OP(v, o_); }  /* row_mirror */           \
+        { uint32_t a_ = v, b_ = v; lanes_swap16(a_, b_); v = OP(a_, b_); }                  \
+        { uint32_t a_ = v, b_ = v; lanes_swap32(a_, b_); v = OP(a_, b_); }                  \
+    } while (0)
+#define CWICK_OP_ADD(a, b) ((a) + (b))
+#define CWICK_OP_MAX(a, b) ((a) > (b) ? (a) : (b))
+#define CWICK_OP_MIN(a, b) ((a) < (b) ? (a) : (b))
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) { CWICK_WAVE_ALLREDUCE(v, CWICK_OP_ADD); return v; }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) { CWICK_WAVE_ALLREDUCE(v, CWICK_OP_MAX); return v; }
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) { CWICK_WAVE_ALLREDUCE(v, CWICK_OP_MIN); return v; }
+// inclusive prefix sum over the lanes of the wave
+__device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v) {
+    v += dpp_u32<0x111, 0xF>(v);     // row_shr:1
+    v += dpp_u32<0x112, 0xF>(v);     // row_shr:2
+    v += dpp_u32<0x114, 0xF>(v);     // row_shr:4
+    v += dpp_u32<0x118, 0xF>(v);     // row_shr:8
+    v += dpp_u32<0x142, 0xA>(v);     // row_bcast:15 into rows 1 and 3
+    v += dpp_u32<0x143, 0xC>(v);     // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// one step of a sum over aligned groups of lanes, every lane of the group ending with the total
+// (a group of `width` lanes whose halves already hold their own totals): DPP inside a row of
+// sixteen, the swaps across rows
+template <int WIDTH>
+__device__ __forceinline__ float group_step_sum(float v) {
+    static_assert(WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "group width");
+    if (WIDTH == 32) return xor16_sum(v);
+    if (WIDTH == 64) return xor32_sum(v);
+    constexpr int CTRL = WIDTH == 2 ? 0xB1 : WIDTH == 4 ? 0x4E : WIDTH == 8 ? 0x141 : 0x140;
+    return v + __builtin_bit_cast(float, dpp_u32<CTRL, 0xF>(__builtin_bit_cast(uint32_t, v)));
+}
+// the maximum over the wave in every lane
 __device__ __forceinline__ float wave_max(float v) {
 #define CWICK_DPP_MAX(ctrl)                                                                                   \
     v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, false)))

@@ -107,13 +107,20 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
                 s[r][j] = d;
             }
         }
-        // butterfly over the LPK lanes of the row: every lane ends with the full dot
+        // the LPK lanes of the row add up their parts, every lane ending with the full dot
+        // (through DPP and lane swaps: no trips through LDS)
 #pragma unroll
-        for (int o = LPK / 2; o > 0; o >>= 1)
+        for (int r = 0; r < GQA_DEC_KB; r++)
 #pragma unroll
-            for (int r = 0; r < GQA_DEC_KB; r++)
-#pragma unroll
-                for (int j = 0; j < GROUP; j++) s[r][j] += __shfl_xor(s[r][j], o, 64);
+            for (int j = 0; j < GROUP; j++) {
+                float t = s[r][j];
+                t = group_step_sum<2>(t);
+                t = group_step_sum<4>(t);
+                t = group_step_sum<8>(t);
+                t = group_step_sum<16>(t);
+                if (LPK == 32) t = group_step_sum<32>(t);
+                s[r][j] = t;
+            }
 #pragma unroll
         for (int r = 0; r < GQA_DEC_KB; r++)
             if (dead[r])
@@ -146,19 +153,31 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
 
     // merge the lane groups of one wave with shuffles (lanes l and l^o hold the
     // same 8 dims of different key subsets) ...
+    // A swap leaves the values of the two lane groups that meet in two registers, the same
+    // pair in every lane: all lanes merge (first, second) in that order.
+    auto meet = [&](float v, int o, float &first, float &second) {
+        uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+        if (o == 16) lanes_swap16(a, b); else lanes_swap32(a, b);
+        first = __builtin_bit_cast(float, a);
+        second = __builtin_bit_cast(float, b);
+    };
 #pragma unroll
     for (int o = LPK; o < 64; o <<= 1) {
 #pragma unroll
         for (int j = 0; j < GROUP; j++) {
-            const float m2 = __shfl_xor(m[j], o, 64);
-            const float l2 = __shfl_xor(l[j], o, 64);
-            const float mx = fmaxf(m[j], m2);
-            const float c1 = mx > -INFINITY ? __expf(m[j] - mx) : 0.0f;
+            float m1, m2, l1, l2;
+            meet(m[j], o, m1, m2);
+            meet(l[j], o, l1, l2);
+            const float mx = fmaxf(m1, m2);
+            const float c1 = mx > -INFINITY ? __expf(m1 - mx) : 0.0f;
             const float c2 = mx > -INFINITY ? __expf(m2 - mx) : 0.0f;
-            l[j] = l[j] * c1 + l2 * c2;
+            l[j] = l1 * c1 + l2 * c2;
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                acc[j][i] = acc[j][i] * c1 + __shfl_xor(acc[j][i], o, 64) * c2;
+            for (int i = 0; i < 8; i++) {
+                float a1, a2;
+                meet(acc[j][i], o, a1, a2);
+                acc[j][i] = a1 * c1 + a2 * c2;
+            }
             m[j] = mx;
         }
     }

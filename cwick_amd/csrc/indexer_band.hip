@@ -269,11 +269,8 @@ indexer_approx_kernel(const uint8_t *__restrict__ keys, const float *__restrict_
         load_keys(it + 4, raw_b, kst_b);
         iteration(it + 2, raw_c, kst_c);
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float other = __shfl_xor(bmax, o, 64);
-        bmax = (other <= bmax) ? bmax : other;
-    }
+    // (never negative: the bit patterns order like the values as unsigned integers, NaNs on top)
+    bmax = __builtin_bit_cast(float, wave_max_u32(__builtin_bit_cast(uint32_t, bmax)));
     if (lane == 0) bmax_sh[wave] = bmax;
     __syncthreads();
     if (tid == 0) {

@@ -34,12 +34,7 @@ constexpr int TOPK_WAVES = TOPK_THREADS / 64;
 // exclusive prefix and writes the block total to *total
 __device__ __forceinline__ uint32_t block_exscan(uint32_t v, uint32_t *sh_wave, uint32_t *total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint32_t inc = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        uint32_t t = __shfl_up(inc, o, 64);
-        if (lane >= o) inc += t;
-    }
+    uint32_t inc = wave_scan_u32(v);
     if (lane == 63) sh_wave[wave] = inc;
     __syncthreads();
     uint32_t wave_off = 0, tot = 0;
@@ -102,12 +97,7 @@ __device__ __forceinline__ void topk_radix_row(const float *__restrict__ sc, int
                 c[j] = hist[255 - (tid * 4 + j)];
                 sum += c[j];
             }
-            uint32_t inc = sum;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                uint32_t t = __shfl_up(inc, o, 64);
-                if (tid >= o) inc += t;
-            }
+            uint32_t inc = wave_scan_u32(sum);
             uint32_t before = inc - sum;   // elements in strictly larger buckets
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -232,12 +222,7 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
                 c[j] = hist[255 - (tid * 4 + j)];
                 sum += c[j];
             }
-            uint32_t inc = sum;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                uint32_t t = __shfl_up(inc, o, 64);
-                if (tid >= o) inc += t;
-            }
+            uint32_t inc = wave_scan_u32(sum);
             uint32_t before = inc - sum;   // elements in strictly larger buckets
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -339,12 +324,7 @@ topk_mw_pick(const uint32_t *__restrict__ slices, int n_wg, int shift, TopkMwSta
             cc[j] = hist[255 - (tid * 4 + j)];
             sum += cc[j];
         }
-        uint32_t inc = sum;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            uint32_t t = __shfl_up(inc, o, 64);
-            if (tid >= o) inc += t;
-        }
+        uint32_t inc = wave_scan_u32(sum);
         uint32_t before = inc - sum;       // elements in strictly larger buckets
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -404,8 +384,7 @@ topk_mw_hist_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
         // these up over the workgroups before it
         const uint32_t dig = (st.prefix >> (32 - 8 * pass)) & 0xFFu;
         uint32_t above = (uint32_t)tid > dig ? own_prev : 0u;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) above += __shfl_xor(above, o, 64);
+        above = wave_sum_u32(above);
         if ((tid & 63) == 0) hist8[tid >> 6] = above;
         __syncthreads();
         if (tid == 0) {
@@ -478,11 +457,8 @@ topk_mw_emit_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int 
         if (above) gt += c;
         if (same) eq += c;
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        gt += __shfl_xor(gt, o, 64);
-        eq += __shfl_xor(eq, o, 64);
-    }
+    gt = wave_sum_u32(gt);
+    eq = wave_sum_u32(eq);
     if (lane == 0) {
         sh_red[0][wave] = gt;
         sh_red[1][wave] = eq;
@@ -559,11 +535,9 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
         v[j] = i < n ? sc[i] : 0.0f;
     }
     float beta = tid < n_beta ? beta_slots[(size_t)row * n_beta + tid] : 0.0f;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float other = __shfl_xor(beta, o, 64);
-        beta = (other <= beta) ? beta : other;                  // NaN sticks
-    }
+    // (bounds are never negative: as unsigned integers their bit patterns order like the values,
+    // with every NaN on top, where it sticks)
+    beta = __builtin_bit_cast(float, wave_max_u32(__builtin_bit_cast(uint32_t, beta)));
     if (lane == 0) sh_beta[tid >> 6] = beta;
     // two digits are enough here: the k-th largest key lies in the bucket [T_lo, T_hi] of the
     // 16-bit prefix (sign, exponent, seven bits of the fraction); at most k-1 keys lie above the
@@ -660,13 +634,9 @@ __device__ __forceinline__ void topk_band_select(const uint32_t (&val)[TOPK_BAND
             mn = val[j] < mn ? val[j] : mn;
             mx = val[j] > mx ? val[j] : mx;
         }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint32_t a = __shfl_xor(mn, o, 64), b = __shfl_xor(mx, o, 64);
-        mn = a < mn ? a : mn;
-        mx = b > mx ? b : mx;
-        cnt += __shfl_xor(cnt, o, 64);
-    }
+    mn = wave_min_u32(mn);
+    mx = wave_max_u32(mx);
+    cnt = wave_sum_u32(cnt);
     if (lane == 0) sh.mn[wave] = mn, sh.mx[wave] = mx, sh.cnt[wave] = cnt;
     __syncthreads();
     cnt = 0u;
@@ -697,12 +667,7 @@ __device__ __forceinline__ void topk_band_select(const uint32_t (&val)[TOPK_BAND
                 c[j] = sh.hist[255 - (tid * 4 + j)];
                 sum += c[j];
             }
-            uint32_t inc = sum;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                uint32_t t = __shfl_up(inc, o, 64);
-                if (tid >= o) inc += t;
-            }
+            uint32_t inc = wave_scan_u32(sum);
             uint32_t before = inc - sum;   // values in strictly larger buckets
 #pragma unroll
             for (int j = 0; j < 4; j++) {
