@@ -301,7 +301,14 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
                        float *__restrict__ cand_score) {   // [batch][cap]: the same scores in list order
     __shared__ float terms[16][65];
     const int b = blockIdx.y, tid = threadIdx.x;
+    int c0 = blockIdx.x * 16;
+    const int j = tid & 15, hg = tid >> 4;                          // candidate, head group
+    // The list entry is fetched next to the row's state, not behind it (one round trip less in
+    // front of the key's bytes): an entry past the end of the list is whatever the workspace
+    // held, so it is clamped to a key of the row; what is computed for it is not stored.
+    int64_t t_guess = cand[(size_t)b * cap + c0 + j];
     const IndexerBandRow st = rows[b];
+    t_guess = t_guess < 0 ? 0 : (t_guess >= n_keys ? n_keys - 1 : t_guess);
     if (indexer_band_failed(st, cap)) {
         // the row did not fit the band: the workgroups of this launch score all of its keys
         // with the exact kernel's code instead
@@ -311,11 +318,13 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
         }
         return;
     }
-    const int c0 = blockIdx.x * 16;
-    if (c0 >= (int)st.n_cand) return;
-    const int j = tid & 15, hg = tid >> 4;                          // candidate, head group
-    const int ci = c0 + j < (int)st.n_cand ? c0 + j : (int)st.n_cand - 1;
-    const int64_t t = cand[(size_t)b * cap + ci];
+    // a list longer than the launch covers in one go (rare) takes further rounds
+    for (; c0 < (int)st.n_cand; c0 += (int)gridDim.x * 16) {
+    int64_t t = t_guess;                                            // (a slot past the end scores some key of the row: not stored)
+    if (c0 != (int)blockIdx.x * 16) {
+        t = cand[(size_t)b * cap + c0 + j];
+        t = t < 0 ? 0 : (t >= n_keys ? n_keys - 1 : t);
+    }
     const uint8_t *krow = keys + (size_t)b * key_bstride + (size_t)t * IB_HD;
     const float ks = kscale[(size_t)b * kscale_bstride + t];
     const uint16_t *qb = q + (size_t)b * ih * IB_HD;
@@ -381,6 +390,8 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
         scores[(size_t)b * n_keys + cand[(size_t)b * cap + c0 + tid]] = s;
         cand_score[(size_t)b * cap + c0 + tid] = s;
     }
+    __syncthreads();                                                // before the next round's terms
+    }
 }
 
 // the approximate scores and the per-workgroup maxima of their error bound (the first stage of
@@ -436,7 +447,12 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     if (!launch_topk_band_classify(scores, batch, n_keys, k, (uint32_t *)ws, beta_slots, n_wg, cand, cap, rows,
                                    hi_count, true, s))
         return 0;
-    indexer_rescore_kernel<<<dim3(cap / 16, batch), 256, 0, s>>>(
+    // Sixteen candidates per workgroup and round.  About one workgroup per CU over all rows: a
+    // list is a few hundred entries, and the launch of workgroups that find nothing to do is what
+    // this kernel's time was mostly made of (256 per row: 7.3 us, 32 per row: 5.4 us for 8 rows).
+    int rescore_wgs = num_cus() / batch;
+    rescore_wgs = rescore_wgs < 8 ? 8 : (rescore_wgs > cap / 16 ? cap / 16 : rescore_wgs);
+    indexer_rescore_kernel<<<dim3(rescore_wgs, batch), 256, 0, s>>>(
         keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, cand, cap, rows, scores, cand_score);
     CWICK_HIP_CALL(hipGetLastError());
     }

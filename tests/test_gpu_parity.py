@@ -386,16 +386,18 @@ def test_dsa_decode_small(hip, orc, n_keys, topk, ih):
     lat.free()
 
 
-@pytest.mark.parametrize("n_keys,topk,copies,take", [(20000, 512, 9, 4), (65536, 2048, 40, 1), (20000, 512, 6, 6)])
-def test_dsa_select_ties_at_the_threshold(hip, orc, n_keys, topk, copies, take):
+@pytest.mark.parametrize("n_keys,topk,copies,take,batch", [(20000, 512, 9, 4, 2), (65536, 2048, 40, 1, 2), (20000, 512, 6, 6, 2),
+                                                             (20000, 512, 1400, 200, 8)])
+def test_dsa_select_ties_at_the_threshold(hip, orc, n_keys, topk, copies, take, batch):
     """The key that closes the selection exists `copies` times (identical rows: identical exact
     scores) and only `take` of the copies fit: the banded path has to rank its candidates by
-    score and then by index, as the reference does."""
-    say("[case] dsa select ties at the threshold", n_keys, topk, copies, take)
-    c = synth.cfg5_dsa(n_keys=n_keys, batch=2, ih=64, topk=topk, nh=128, seed=1300 + copies)
+    score and then by index, as the reference does.  The last case makes the candidate list of
+    each of eight rows longer than one round of the rescoring kernel covers."""
+    say("[case] dsa select ties at the threshold", n_keys, topk, copies, take, batch)
+    c = synth.cfg5_dsa(n_keys=n_keys, batch=batch, ih=64, topk=topk, nh=128, seed=1300 + copies)
     ikeys = c["ikeys"].copy(); ikscale = c["ikscale"].copy()
     g = synth.rng(77 + copies)
-    for b in range(2):
+    for b in range(batch):
         sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], ikeys[b], ikscale[b], nthreads=0)
         order = np.lexsort((np.arange(n_keys), -sc.astype(np.float64)))
         # rank topk - take (0-based) is the first copy's rank: `take` copies end the selection
@@ -404,13 +406,13 @@ def test_dsa_select_ties_at_the_threshold(hip, orc, n_keys, topk, copies, take):
         dst = g.choice(order[topk + 50:], size=copies - 1, replace=False)
         ikeys[b, dst] = ikeys[b, src]
         ikscale[b, dst] = ikscale[b, src]
-    ik = hip.IndexKeys(2, n_keys)
-    lat = hip.LatentCache(2, n_keys)
-    for b in range(2):
+    ik = hip.IndexKeys(batch, n_keys)
+    lat = hip.LatentCache(batch, n_keys)
+    for b in range(batch):
         ik.write(b, 0, ikeys[b], ikscale[b])
         lat.write(b, 0, c["rows"][b], c["scales"][b])
     out, sel = hip.dsa_decode(ik, lat, 0, 1, n_keys, c["q_idx"], c["w"], topk, c["q"], c["scale"])
-    for b in range(2):
+    for b in range(batch):
         sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], ikeys[b], ikscale[b], nthreads=0)
         rsel = orc.topk_contract(sc, topk)
         T = np.sort(sc)[::-1][topk - 1]
