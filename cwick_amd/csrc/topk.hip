@@ -578,7 +578,9 @@ topk_mw_classify_kernel(float *__restrict__ scores, int64_t n, int64_t k, int n_
     uint32_t my_first = 0u;
     const uint32_t mine = (uint32_t)__builtin_popcount(is_cand);
     if (mine) my_first = atomicAdd(wg_count, mine);
-    if (n_hi) atomicAdd(wg_hi, n_hi);
+    // (one atomic per wave: a few dozen on one address from one instruction queue up)
+    n_hi = wave_sum_u32(n_hi);
+    if (lane == 0 && n_hi) atomicAdd(wg_hi, n_hi);
     __syncthreads();
     if (tid == 0) {
         *wg_base = *wg_count ? atomicAdd(&rows[row].n_cand, *wg_count) : 0u;
@@ -727,10 +729,11 @@ topk_band_finish_kernel(const float *__restrict__ scores, int64_t n, int64_t k, 
         return;
     }
     const int n_cand = (int)st.n_cand;
-    if (tid == 0) sh_hi = 0u, sh_before = 0u;
-    __syncthreads();
-    if (tid < n_wg) atomicAdd(&sh_hi, hi_part);
-    if (tid < wg) atomicAdd(&sh_before, hi_part);
+    static_assert(TOPK_MW_MAX_WGS <= 64, "the first wave holds a count per stretch");
+    if (tid < 64) {                                             // the first wave adds up the stretches' counts
+        const uint32_t all = wave_sum_u32(hi_part), before = wave_sum_u32(tid < wg ? hi_part : 0u);
+        if (tid == 0) sh_hi = all, sh_before = before;
+    }
     uint32_t key[TOPK_BAND_EPT], inv[TOPK_BAND_EPT], live = 0u;
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++) {
@@ -759,7 +762,9 @@ topk_band_finish_kernel(const float *__restrict__ scores, int64_t n, int64_t k, 
 #pragma unroll
     for (int j = 0; j < TOPK_BAND_EPT; j++)
         if ((live >> j & 1u) && (int64_t)idx[j] < base && chosen(key[j], inv[j])) earlier++;
-    if (earlier) atomicAdd(&sh_before, earlier);
+    // (added up per wave first: hundreds of atomics on one address would queue up)
+    earlier = wave_sum_u32(earlier);
+    if (lane == 0 && earlier) atomicAdd(&sh_before, earlier);
     // own keys: +inf is in, -inf is out, anything else is a candidate with its exact score.
     // Element (j, tid) is index base + 1024 j + tid: the order of the workgroup is (j, wave, lane)
     uint64_t m[KPT];
