@@ -24,8 +24,9 @@
 //   the accumulating waves (and the scorers, for their sums) bring everything to the common
 //   maximum.  Each scoring lane keeps the sum of its own keys; the sums meet once, after the loop.
 //   Tiles are copied global -> LDS by global_load_lds (no registers) into four stages.  Tile 0 is
-//   fetched by all twelve waves at kernel start, tiles 1 and 2 by the two waves that have no part
-//   in the preparation of Q; from step 0 on every wave copies its share of tile t+3 during step t
+//   fetched by all twelve waves at kernel start, tile 1 behind it by the two waves that have no
+//   part in the preparation of Q, tile 2 by the value waves behind the first barrier; from step 0
+//   on every wave copies its share of tile t+3 during step t
 //   (three sixteen-byte columns of the 64 rows, plus a scale block for five of the waves): the
 //   value waves at the top of the step, the scoring waves at the end of theirs, when they would
 //   otherwise wait at the barrier.  The copies are issued from inline assembly and the barrier
@@ -302,19 +303,46 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         if (wave < NBLK) dma4(sp + 4 * wave, tile_off + SC_OFF + (uint32_t)wave * (TK * 4));
         if (SEL && wave == 0) mark(r, tile_off);
     };
-    auto whole = [&](int r, uint32_t tile_off) {
+    // pieces first, first + stride, ... of a tile
+    auto part = [&](int r, uint32_t tile_off, int first, int stride) {
         const uint64_t rp = row_ptr(r), sp = sc_ptr(r);
 #pragma unroll
-        for (int pc = 0; pc < NCOL + NBLK; pc++) piece(pc, rp, sp, tile_off);
-        if (SEL) mark(r, tile_off);
+        for (int pc = 0; pc < NCOL + NBLK; pc++)
+            if (pc >= first && (pc - first) % stride == 0) piece(pc, rp, sp, tile_off);
+        if (SEL && first == 0) mark(r, tile_off);
     };
-    // Tile 0 is fetched by everybody at once; then waves 10 and 11, which have no part in the
-    // preparation of Q, fetch tiles 1 and 2.  From step 0 on tile t+3 is fetched during step t,
-    // every wave its share.
-    if (n_tiles > 0) share(row_of(0), lds0);
-    const bool fetched_whole = (wave == 10 && n_tiles > 1) || (wave == 11 && n_tiles > 2);
-    if (wave == 10 && n_tiles > 1) whole(row_of(1), lds0 + TILE_B);
-    if (wave == 11 && n_tiles > 2) whole(row_of(2), lds0 + 2 * TILE_B);
+    // Tile 0 is fetched by everybody at once, and tile 1 right behind it by waves 10 and 11,
+    // which have no part in the preparation of Q (the memory pipeline takes a copy every few
+    // dozen cycles while every workgroup starts cold, and the first tiles of all workgroups are
+    // a third of the cache: the memory system has to start on them at once).  Tile 2 follows
+    // behind the first barrier, a quarter from each value wave while the scoring waves read
+    // their Q back: two waves that issued tiles 1 and 2 whole held that barrier back by
+    // 3 000 cycles.  From step 0 on tile t+3 is fetched during step t, every wave its share.
+    int r12[2] = {row_of(1), row_of(2)};
+    // (list entries are loads: in before the first copy goes out, or the wait for them would
+    // sit out the copies)
+    int r0 = row_of(0);
+    if (SEL) asm volatile("" : "+v"(r0), "+v"(r12[0]), "+v"(r12[1])::"memory");
+    // The query goes first: the copies of a compute unit queue up in one memory pipeline, and a
+    // Q load behind forty of them arrives thousands of cycles late (the preparation of Q is
+    // what the first barrier waits for).  Its loads are written in assembly like the copies, so
+    // that the wait for them can leave the copies issued behind them in flight (a wait that the
+    // compiler places counts only the loads it knows).
+    u32x4 qraw[4];            // (no initialiser and one definition: a second one would make the compiler copy registers whose loads are still in flight)
+    if (wave < 10) {
+        const int hhu = wave / 5, b = wave % 5;
+        int head = hb * HW + 16 * hhu + n;
+        if (head >= p.nh) head = p.nh - 1;
+        const uint16_t *src = p.q + ((size_t)y * p.nh + head) * KDIM + (b < 4 ? 128 * b + 32 * g : 512 + 32 * (g & 1));
+        asm volatile("global_load_dwordx4 %0, %4, off\n\t"
+                     "global_load_dwordx4 %1, %4, off offset:16\n\t"
+                     "global_load_dwordx4 %2, %4, off offset:32\n\t"
+                     "global_load_dwordx4 %3, %4, off offset:48"
+                     : "=&v"(qraw[0]), "=&v"(qraw[1]), "=&v"(qraw[2]), "=&v"(qraw[3]) : "v"(src) : "memory");
+    }
+    if (n_tiles > 0) share(r0, lds0);
+    const bool half_of_1 = wave >= 10 && n_tiles > 1;
+    if (half_of_1) part(r12[0], lds0 + TILE_B, wave == 10 ? 0 : 1, 2);      // 21 pieces or 20
 
     // ---- Q for 2 x 16 heads as two E4M3 terms per 32-dim block with one E8M0 scale per head and
     // 128-dim block (the hardware pairs the scale of lane (n, g) with k-elements that live in other
@@ -327,15 +355,17 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         QPark *park = reinterpret_cast<QPark *>(&sm.tile[NST - 1]);
         if (wave < 10) {
             const int u = wave;
-            const int hhu = u / 5, b = u % 5;
-            int head = hb * HW + 16 * hhu + n;
-            if (head >= p.nh) head = p.nh - 1;
-            const uint16_t *qrow = p.q + ((size_t)y * p.nh + head) * KDIM;
-            const uint16_t *src = qrow + (b < 4 ? 128 * b + 32 * g : 512 + 32 * (g & 1));
+            const int b = u % 5;
+            // the share of tile 0 (three columns, and a scale block for the first five waves) stays in flight
+            if (n_tiles <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else if (wave < NBLK) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+            // the registers count as written here, behind the waits
+            asm volatile("" : "+v"(qraw[0]), "+v"(qraw[1]), "+v"(qraw[2]), "+v"(qraw[3])::"memory");
             float qv[32];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const u32x4 w = *(const u32x4 *)(src + 8 * c);
+                const u32x4 w = qraw[c];
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
                     qv[8 * c + 2 * d] = bf16lo_to_f32(w[d]);
@@ -371,14 +401,16 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
             }
             qp->sc[lane] = 127 + s;
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // tile 0 has landed (this wave's share)
-        } else if (fetched_whole) {
-            // the share of tile 0 was issued before the 41 copies of tile 1 or 2, which stay in flight
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NCOL + NBLK) : "memory");
+        } else if (half_of_1) {
+            // the share of tile 0 was issued before the copies of tile 1, which stay in flight
+            if (wave == 10) asm volatile("s_waitcnt vmcnt(21)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         LDS_BARRIER();
     }
+    static_assert(NCOL + NBLK == 41, "the counts of copies in flight above and below");
 
     const float c0 = p.scale * 1.44269504088896340736f;   // scores in log2 units
     float m_ref[2] = {-INFINITY, -INFINITY};          // of head 16 h2 + n; every wave tracks the same values
@@ -542,6 +574,9 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         if (g == 0) lsum[(hh * 16 + n) * 4 + kb] = ls;
         LDS_BARRIER();
     } else {
+        // tile 2 (stage 2; Q is parked in the last stage and the exchange area): pieces cw, cw + 4, ...
+        const bool quarter_of_2 = n_tiles > 2;
+        if (quarter_of_2) part(r12[1], lds0 + 2 * TILE_B, cw, 4);           // 11 pieces for cw = 0, else 10
         LDS_BARRIER();                                // before copies or weights land in the park area
         f32x4 oacc[2][8];                                 // [head half][dim block]: dims 128 cw + 16 j + 4 g + i, head n
 #pragma unroll
@@ -678,10 +713,13 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 }
             }
             // tile t+2 must be whole at the next barrier; the share of tile t+3 issued in this
-            // step (four copies by waves 8, three by the others) may stay in flight.  Wave 11 has the
-            // whole of tile 2 in flight in step -1: it is needed one step later than tile 1.
+            // step (three copies) may stay in flight, and in step -1 this wave's quarter of tile 2,
+            // which is needed one step later than tile 1
             if (do_copy) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-            else if (!(t < 0 && wave == 11)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else if (t < 0 && quarter_of_2) {
+                if (cw == 0) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+            } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             LDS_BARRIER();
         }
 
