@@ -138,6 +138,7 @@ int launch_dequant_latent(const uint8_t *rows, const float *scales, int64_t n, f
 int launch_dequant_ikeys(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
 int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);
 int launch_e4m3_table(float *out256_dev, hipStream_t s);
+int launch_lane_ops(const uint32_t *in64_dev, uint32_t *out832_dev, hipStream_t s);
 int run_probe_hbm_read(size_t bytes, int reps, double *gbps);
 int run_probe_mfma(int kind, int reps, double *tflops);
 

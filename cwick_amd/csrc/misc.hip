@@ -103,6 +103,32 @@ int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s)
     return 1;
 }
 
+// one wave: every lane-exchange primitive of common.hpp on the 64 words of `in`
+__global__ void __launch_bounds__(64) lane_ops_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out) {
+    const int l = threadIdx.x;
+    const uint32_t v = in[l];
+    const float f = __builtin_bit_cast(float, (v & 0x007FFFFFu) | 0x3F800000u);      // in [1, 2)
+    out[l] = wave_sum_u32(v);
+    out[64 + l] = wave_max_u32(v);
+    out[128 + l] = wave_min_u32(v);
+    out[192 + l] = wave_scan_u32(v);
+    out[256 + l] = __builtin_bit_cast(uint32_t, wave_max(f));
+    out[320 + l] = __builtin_bit_cast(uint32_t, xor16_max(f));
+    out[384 + l] = __builtin_bit_cast(uint32_t, xor32_max(f));
+    out[448 + l] = __builtin_bit_cast(uint32_t, xor16_sum(f));
+    out[512 + l] = __builtin_bit_cast(uint32_t, xor32_sum(f));
+    out[576 + l] = __builtin_bit_cast(uint32_t, group_step_sum<2>(f));
+    out[640 + l] = __builtin_bit_cast(uint32_t, group_step_sum<4>(group_step_sum<2>(f)));
+    out[704 + l] = __builtin_bit_cast(uint32_t, group_step_sum<8>(group_step_sum<4>(group_step_sum<2>(f))));
+    out[768 + l] = __builtin_bit_cast(uint32_t, group_step_sum<16>(group_step_sum<8>(group_step_sum<4>(group_step_sum<2>(f)))));
+}
+
+int launch_lane_ops(const uint32_t *in64_dev, uint32_t *out832_dev, hipStream_t s) {
+    lane_ops_kernel<<<1, 64, 0, s>>>(in64_dev, out832_dev);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
 int launch_e4m3_table(float *out256_dev, hipStream_t s) {
     e4m3_table_kernel<<<1, 256, 0, s>>>(out256_dev);
     CWICK_HIP_CALL(hipGetLastError());

@@ -1151,4 +1151,19 @@ int cwick_hip_e4m3_table(float *out256) {
     return st.out(out256, d, 1024) && st.wait() ? 1 : 0;
 }
 
+int cwick_hip_lane_ops(const uint32_t *in64, uint32_t *out832) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    CWICK_REQUIRE(in64 && out832, "lane_ops: null argument");
+    std::lock_guard<std::mutex> lk(g_free_mu);
+    if (!g_free_ctx.stream) CWICK_REQUIRE(g_free_ctx.init(), "lane_ops: no stream");
+    Stager st(g_free_ctx, 256 + 832 * 4 + 256);
+    CWICK_REQUIRE(st.ok, "lane_ops: staging allocation failed");
+    const uint32_t *din = st.in(in64, 256);
+    uint32_t *dout = st.room<uint32_t>(832 * 4);
+    CWICK_REQUIRE(din, "lane_ops: upload failed");
+    if (!launch_lane_ops(din, dout, g_free_ctx.stream)) return 0;
+    return st.out(out832, dout, 832 * 4) && st.wait() ? 1 : 0;
+}
+
 }  // extern "C"

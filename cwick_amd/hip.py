@@ -99,6 +99,7 @@ SIGNATURES = {
     "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
     "cwick_hip_probe_mfma": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
+    "cwick_hip_lane_ops": (_int, [_vp, _vp]),
     "cwick_hip_prof_enable": (None, [_int]),
     "cwick_hip_prof_reset": (None, []),
     "cwick_hip_prof_read": (_int, [_int, C.POINTER(C.c_double), C.POINTER(_i64)]),
@@ -460,6 +461,15 @@ def probe_mfma(kind=0, reps=3):
     v = C.c_double(0.0)
     _check(lib().cwick_hip_probe_mfma(kind, reps, C.byref(v)), "probe_mfma")
     return v.value
+
+
+def lane_ops(words):
+    """The wave-level exchange primitives applied to 64 words: [13][64] uint32 (see cwick_hip.h)."""
+    w = np.ascontiguousarray(words, dtype=np.uint32)
+    assert w.shape == (64,)
+    out = np.empty((13, 64), np.uint32)
+    _check(lib().cwick_hip_lane_ops(w.ctypes.data, out.ctypes.data), "lane_ops")
+    return out
 
 
 def e4m3_table():

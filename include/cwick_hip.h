@@ -469,6 +469,16 @@ int cwick_hip_probe_mfma(int kind, int reps, double *tflops);
  * bytes with the conversion instruction the kernels use into out256 (host). */
 int cwick_hip_e4m3_table(float *out256);
 
+/* Device-side check of the lane exchanges the kernels are built on (sums, maxima and prefix sums
+ * over a wave through DPP and lane swaps instead of LDS): one wave applies each of them to the 64
+ * words of in64 (host); out832 (host) receives thirteen results of 64 words: sum, maximum, minimum
+ * and inclusive prefix sum of the words as unsigned integers; then, on the floats
+ * 1.m (m = the low 23 bits of a word), the maximum over the wave, the maximum and the sum over
+ * lanes l and l ^ 16, over l and l ^ 32, and the sums over aligned groups of 2, 4, 8 and 16
+ * lanes.  No counterpart in the reference (its reductions are NEON lanes and pthread slices);
+ * used by the parity tests. */
+int cwick_hip_lane_ops(const uint32_t *in64, uint32_t *out832);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,36 @@ def say(*a):
 
 
 # ------------------------------------------------------------------ codecs
+def test_lane_exchange_primitives(hip):
+    """Sums, maxima and prefix sums over a wave (DPP inside a row of sixteen lanes, lane swaps
+    across rows) against numpy, bit for bit: every kernel's reductions are built on them."""
+    say("[case] lane exchange primitives")
+    g = synth.rng(4242)
+    for rep in range(8):
+        w = g.integers(0, 1 << 32 if rep % 2 else 100000, size=64, dtype=np.uint64).astype(np.uint32)
+        if rep == 7:
+            w[:] = 0
+            w[37] = 0xFFFFFFFF
+        got = hip.lane_ops(w)
+        f = ((w & 0x007FFFFF) | 0x3F800000).view(np.float32)
+        assert np.all(got[0] == np.uint32(w.astype(np.uint64).sum() & 0xFFFFFFFF))
+        assert np.all(got[1] == w.max()) and np.all(got[2] == w.min())
+        assert np.array_equal(got[3], (np.cumsum(w.astype(np.uint64)) & 0xFFFFFFFF).astype(np.uint32))
+        assert np.all(got[4].view(np.float32) == f.max())
+        l = np.arange(64)
+        assert np.array_equal(got[5].view(np.float32), np.maximum(f, f[l ^ 16]))
+        assert np.array_equal(got[6].view(np.float32), np.maximum(f, f[l ^ 32]))
+        # a + b in fp32 is the same whichever side a lane stands on
+        assert np.array_equal(got[7].view(np.float32), f + f[l ^ 16])
+        assert np.array_equal(got[8].view(np.float32), f + f[l ^ 32])
+        s2 = f + f[l ^ 1]
+        s4 = s2 + s2[l ^ 2]
+        s8 = s4 + s4[l ^ 4]
+        s16 = s8 + s8[l ^ 8]
+        for row, want in ((9, s2), (10, s4), (11, s8), (12, s16)):
+            assert np.array_equal(got[row].view(np.float32), want), "group sum %d" % row
+
+
 def test_e4m3_hardware_decode_matches_table(hip, orc):
     say("[case] e4m3 table")
     got = hip.e4m3_table()
