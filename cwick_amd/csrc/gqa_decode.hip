@@ -183,7 +183,7 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
     }
     // ... and the waves of the workgroup through LDS
     constexpr int NW = GQA_DEC_THREADS / 64;
-    __shared__ float sh_acc[NW][GROUP][HD];
+    __shared__ __attribute__((aligned(16))) float sh_acc[NW][GROUP][HD];
     __shared__ float sh_m[NW][GROUP], sh_l[NW][GROUP];
     const int wave = tid >> 6;
     if ((tid & 63) < LPK) {
@@ -198,24 +198,31 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
         }
     }
     __syncthreads();
-    for (int idx = tid; idx < GROUP * HD; idx += GQA_DEC_THREADS) {
-        const int j = idx / HD, d = idx % HD;
+    // a thread takes four consecutive dims of one head: the waves' weights once per four values,
+    // the values in 16-byte LDS reads, two 8-byte stores
+    for (int i4 = tid; i4 < GROUP * HD / 4; i4 += GQA_DEC_THREADS) {
+        const int j = i4 / (HD / 4), d = (i4 % (HD / 4)) * 4;
         float mx = -INFINITY;
 #pragma unroll
         for (int w = 0; w < NW; w++) mx = fmaxf(mx, sh_m[w][j]);
-        float a = 0.0f, ls = 0.0f;
+        f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
+        float ls = 0.0f;
         if (mx > -INFINITY) {
 #pragma unroll
             for (int w = 0; w < NW; w++) {
                 const float c = __expf(sh_m[w][j] - mx);   // exp(-inf) = 0 for idle waves
-                a += sh_acc[w][j][d] * c;
+                const f32x4 t = *(const f32x4 *)&sh_acc[w][j][d];
+#pragma unroll
+                for (int r = 0; r < 4; r++) a[r] += t[r] * c;
                 ls += sh_l[w][j] * c;
             }
         }
         const int h = g * GROUP + j;
         // written through: the merge kernel reads it from other XCDs, and a dirty line would be
         // written back at the end of this kernel
-        __hip_atomic_store(&part_acc[((size_t)split * n_heads + h) * HD + d], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        uint64_t *dst = (uint64_t *)&part_acc[((size_t)split * n_heads + h) * HD + d];
+        __hip_atomic_store(dst, __builtin_bit_cast(uint64_t, (f32x2){a[0], a[1]}), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(dst + 1, __builtin_bit_cast(uint64_t, (f32x2){a[2], a[3]}), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (d == 0) {
             part_ml[((size_t)split * n_heads + h) * 2 + 0] = mx;
             part_ml[((size_t)split * n_heads + h) * 2 + 1] = ls;
