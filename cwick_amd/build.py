@@ -17,7 +17,7 @@ OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libcwick_hip.so")
 
 SOURCES = ["runtime.hip", "misc.hip", "gqa_decode.hip", "gqa_prefill.hip", "mla_roles.hip",
-           "indexer.hip", "indexer_band.hip", "topk.hip", "probe.hip", "prep.hip", "mla_prefill64.hip"]
+           "indexer.hip", "indexer_band.hip", "topk.hip", "probe.hip", "prep.hip", "mla_prefill64.hip", "mm_select.hip"]
 
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
           "-Wall", "-Wno-unused-function",

@@ -133,6 +133,9 @@ int launch_ikeys_pool(const float *tail_k, const float *tail_g, const uint16_t *
                       hipStream_t s);
 int launch_candidate_select(const float *scores, int batch, int64_t n, int block, int64_t topk_blocks, uint8_t *cand,
                             hipStream_t s);
+int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0, int index_heads,
+                     int index_dim, int block, int keep_blocks, float *scores, int64_t score_stride,
+                     int32_t *blk_out, int32_t *sel, int64_t max_sel, int32_t *n_sel, hipStream_t s);
 int launch_candidate_apply(float *scores, const uint8_t *cand, int batch, int64_t n, hipStream_t s);
 int launch_dequant_latent(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
 int launch_dequant_ikeys(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);

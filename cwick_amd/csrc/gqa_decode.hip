@@ -35,14 +35,17 @@ __global__ void __launch_bounds__(GQA_DEC_THREADS)
 gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
                         const uint16_t *__restrict__ Q, int64_t n_keys, int n_kv_heads,
                         const int32_t *__restrict__ sel, int64_t n_rows,
-                        int keys_per_split, float scale,
+                        int keys_per_split, int kv_shift, float scale,
                         float *__restrict__ part_acc,   // [n_splits][n_heads][HD]
                         float *__restrict__ part_ml) {  // [n_splits][n_heads][2]
     constexpr int LPK = HD / 8;                 // lanes per key row
     constexpr int NGRP = GQA_DEC_THREADS / LPK; // lane groups per workgroup
+    // a kv head whose group is larger than GROUP is served by 1 << kv_shift workgroups, each with
+    // GROUP of its query heads
     const int g = blockIdx.y;
+    const int gk = g >> kv_shift;
     const int split = blockIdx.x;
-    const int n_heads = n_kv_heads * GROUP;
+    const int n_heads = (n_kv_heads << kv_shift) * GROUP;
     const int tid = threadIdx.x;
     const int sub = tid % LPK;                  // which 8 dims of the row
     const int grp = tid / LPK;                  // which lane group
@@ -71,8 +74,8 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
         for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
     }
 
-    const uint16_t *Kg = K + (size_t)g * HD + sub * 8;
-    const uint16_t *Vg = V + (size_t)g * HD + sub * 8;
+    const uint16_t *Kg = K + (size_t)gk * HD + sub * 8;
+    const uint16_t *Vg = V + (size_t)gk * HD + sub * 8;
 
     for (int64_t base = k_begin + (int64_t)grp * GQA_DEC_KB; base < k_end;
          base += (int64_t)NGRP * GQA_DEC_KB) {
@@ -233,15 +236,16 @@ gqa_decode_split_kernel(const uint16_t *__restrict__ K, const uint16_t *__restri
 template <int HD, int GROUP>
 static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int n_kv_heads,
                           const int32_t *sel, int64_t n_rows, const uint16_t *q, float scale, float *out,
-                          hipStream_t s) {
-    const int n_heads = n_kv_heads * GROUP;
+                          hipStream_t s, int kv_shift = 0) {
+    const int n_units = n_kv_heads << kv_shift;            // (kv head, GROUP query heads) pairs
+    const int n_heads = n_units * GROUP;
     constexpr int LPK = HD / 8, NGRP = GQA_DEC_THREADS / LPK;
     constexpr int step = NGRP * GQA_DEC_KB;   // rows one workgroup consumes per iteration
     // enough workgroups for ~2 per CU, each at least one full step
     const char *env = getenv("CWICK_HIP_GQA_WG_PER_CU");
     int per_cu = env ? atoi(env) : 2;
     if (per_cu < 1 || per_cu > 8) per_cu = 2;
-    int64_t want = (int64_t)per_cu * num_cus() / n_kv_heads;
+    int64_t want = (int64_t)per_cu * num_cus() / n_units;
     if (want < 1) want = 1;
     if (want > MERGE_MAX_SPLITS) want = MERGE_MAX_SPLITS;
     int64_t per = (n_keys + want - 1) / want;
@@ -255,8 +259,8 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     float *part_acc = (float *)ws, *part_ml = (float *)(ws + acc_bytes);
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_DECODE, s);
-        gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_kv_heads), GQA_DEC_THREADS, 0, s>>>(
-            k, v, q, n_keys, n_kv_heads, sel, n_rows, (int)per, scale, part_acc, part_ml);
+        gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_units), GQA_DEC_THREADS, 0, s>>>(
+            k, v, q, n_keys, n_kv_heads, sel, n_rows, (int)per, kv_shift, scale, part_acc, part_ml);
     }
     CWICK_HIP_CALL(hipGetLastError());
     {
@@ -286,7 +290,10 @@ int launch_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, int 
     CASE(256, 1); CASE(256, 2); CASE(256, 4); CASE(256, 8);
     CASE(128, 1); CASE(128, 2); CASE(128, 4); CASE(128, 8);
 #undef CASE
-    set_error("gqa_decode: head_dim %d with group %d is not supported (head_dim 128/256, group 1/2/4/8)",
+    // sixteen query heads per kv head (the block-sparse family's 64/4): two workgroups of eight
+    if (group == 16 && head_dim == 256) return run_gqa_decode<256, 8>(k, v, n_keys, n_kv_heads, sel, n_rows, q, scale, out, s, 1);
+    if (group == 16 && head_dim == 128) return run_gqa_decode<128, 8>(k, v, n_keys, n_kv_heads, sel, n_rows, q, scale, out, s, 1);
+    set_error("gqa_decode: head_dim %d with group %d is not supported (head_dim 128/256, group 1/2/4/8/16)",
               head_dim, group);
     return 0;
 }

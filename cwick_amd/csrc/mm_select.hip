@@ -1,0 +1,180 @@
+// Block selection of the block-sparse GQA decode (the MiniMax family of the reference).
+//
+// Replaces, for one query or a chunk of consecutive ones, mm_index_scores (src/mm_model.c:
+// 1764-1780), mm_select_blocks (:1733-1761) and the loop that writes the chosen blocks out as
+// positions (:1969-1976).  What leaves is a position list per query, padded with -1, that
+// launch_gqa_decode takes as its `sel`: the whole selection stays on the device.
+//
+//   1. mm_index_scores_kernel   one thread per position: for every index head the dot of the
+//      head's fp32 query with the position's bf16 key, a fused multiply-add per dimension in
+//      dimension order from zero (the reference's serial loop), ReLU, the heads added in head
+//      order.  The query sits in LDS and is read as a broadcast; a thread streams its own
+//      256-byte key row in 16-byte pieces.
+//   2. mm_blockmax_kernel       one wave per block: the largest score inside the block, started
+//      from -1e30 like the reference; blocks past a query's last one get -inf so that rows of
+//      a chunk with different block counts share one top-k launch.
+//   3. launch_topk              the `keep` best blocks, lowest index first among equal maxima
+//      (the reference's heap makes that choice on tie-free input).
+//   4. mm_expand_kernel         adds block limit / block when it is not among the chosen (for a
+//      limit that is a multiple of the block size this is a block without a written position,
+//      which contributes nothing -- the reference's rule, kept as it is) and writes the
+//      positions: chosen blocks are full except the last, so position p of the list is
+//      block[p / block] * block + p % block, or -1 past the limit.
+#include "common.hpp"
+
+namespace cwick {
+namespace {
+
+constexpr int MM_THREADS = 256;
+constexpr int MM_MAX_HEADS = 8;
+constexpr int MM_MAX_DIM = 512;
+
+__global__ void __launch_bounds__(MM_THREADS)
+mm_index_scores_kernel(const uint16_t *__restrict__ keys, const float *__restrict__ iq, int64_t limit0, int ih, int id,
+                       float *__restrict__ scores, int64_t score_stride) {
+    __shared__ __attribute__((aligned(16))) float qs[MM_MAX_HEADS * MM_MAX_DIM];
+    const int row = blockIdx.y;
+    const int64_t limit = limit0 + row;
+    if ((int64_t)blockIdx.x * MM_THREADS >= limit) return;          // the whole workgroup: before any barrier
+    const float *q = iq + (size_t)row * ih * id;
+    for (int i = threadIdx.x; i < ih * id; i += MM_THREADS) qs[i] = q[i];
+    __syncthreads();
+    const int64_t s = (int64_t)blockIdx.x * MM_THREADS + threadIdx.x;
+    const int64_t sc = s < limit ? s : limit - 1;                   // threads past the end read the last row
+    const u32x4 *kp = (const u32x4 *)(keys + (size_t)sc * id);
+    float d[MM_MAX_HEADS];
+#pragma unroll
+    for (int h = 0; h < MM_MAX_HEADS; h++) d[h] = 0.0f;
+    const int chunks = id / 8;
+    u32x4 kw = kp[0];
+    for (int c = 0; c < chunks; c++) {
+        const u32x4 cur = kw;
+        if (c + 1 < chunks) kw = kp[c + 1];
+        float kf[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            kf[2 * i] = bf16lo_to_f32(cur[i]);
+            kf[2 * i + 1] = bf16hi_to_f32(cur[i]);
+        }
+#pragma unroll
+        for (int h = 0; h < MM_MAX_HEADS; h++) {
+            if (h < ih) {                                           // uniform
+                const f32x4 qa = *(const f32x4 *)(qs + h * id + c * 8);
+                const f32x4 qb = *(const f32x4 *)(qs + h * id + c * 8 + 4);
+#pragma unroll
+                for (int i = 0; i < 4; i++) d[h] = __builtin_fmaf(qa[i], kf[i], d[h]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) d[h] = __builtin_fmaf(qb[i], kf[4 + i], d[h]);
+            }
+        }
+    }
+    float tot = 0.0f;
+#pragma unroll
+    for (int h = 0; h < MM_MAX_HEADS; h++)
+        if (h < ih && d[h] > 0.0f) tot = tot + d[h];
+    if (s < limit) scores[(size_t)row * score_stride + s] = tot;
+}
+
+__global__ void __launch_bounds__(MM_THREADS)
+mm_blockmax_kernel(const float *__restrict__ scores, int64_t score_stride, int64_t limit0, int bs, int64_t nblk_max,
+                   float *__restrict__ bsc) {
+    const int lane = threadIdx.x & 63;
+    const int64_t b = (int64_t)blockIdx.x * (MM_THREADS / 64) + (threadIdx.x >> 6);
+    const int row = blockIdx.y;
+    if (b >= nblk_max) return;
+    const int64_t limit = limit0 + row;
+    const int64_t lo = b * bs, hi = lo + bs < limit ? lo + bs : limit;
+    float mx = lo < limit ? -1e30f : -INFINITY;
+    const float *sc = scores + (size_t)row * score_stride;
+    for (int64_t t = lo + lane; t < hi; t += 64) mx = fmaxf(mx, sc[t]);
+    mx = wave_max(mx);
+    if (lane == 0) bsc[(size_t)row * nblk_max + b] = mx;
+}
+
+__global__ void __launch_bounds__(MM_THREADS)
+mm_expand_kernel(const int32_t *__restrict__ blk, int kb, int64_t limit0, int bs, int32_t *__restrict__ blk_out,
+                 int32_t *__restrict__ sel, int64_t max_sel, int32_t *__restrict__ n_sel) {
+    __shared__ uint32_t sh_nv, sh_has;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int64_t limit = limit0 + row;
+    const int64_t nblk = (limit + bs - 1) / bs;
+    const int32_t newest = (int32_t)(limit / bs);
+    const int32_t *mine = blk + (size_t)row * kb;
+    if (tid == 0) sh_nv = 0, sh_has = 0;
+    __syncthreads();
+    // the chosen blocks come in ascending order, blocks this query does not have (and the -1
+    // padding of a short row) after the ones it has: the valid entries are a prefix
+    for (int j0 = 0; j0 < kb; j0 += MM_THREADS) {
+        const int j = j0 + tid;
+        const int32_t b = j < kb ? mine[j] : -1;
+        const uint32_t ok = b >= 0 && b < nblk;
+        const uint32_t cnt = wave_sum_u32(ok), has = wave_sum_u32(ok && b == newest);
+        if ((tid & 63) == 0 && cnt) atomicAdd(&sh_nv, cnt);
+        if ((tid & 63) == 0 && has) atomicAdd(&sh_has, has);
+    }
+    __syncthreads();
+    const int nv = (int)sh_nv;
+    const int nb = nv + (sh_has ? 0 : 1);
+    if (blk_out)
+        for (int j = tid; j <= kb; j += MM_THREADS)
+            blk_out[(size_t)row * (kb + 1) + j] = j < nv ? mine[j] : j < nb ? newest : -1;
+    // every block of the list but its last is full
+    for (int64_t p = tid; p < max_sel; p += MM_THREADS) {
+        const int64_t j = p / bs;
+        int64_t pos = -1;
+        if (j < nb) {
+            const int64_t b = j < nv ? mine[j] : newest;
+            pos = b * bs + (p - j * bs);
+            if (pos >= limit) pos = -1;
+        }
+        sel[(size_t)row * max_sel + p] = (int32_t)pos;
+    }
+    if (n_sel && tid == 0) {
+        const int64_t last = nb - 1 < nv ? mine[nb - 1] : newest;
+        int64_t in_last = limit - last * bs;
+        in_last = in_last < 0 ? 0 : in_last > bs ? bs : in_last;
+        const int64_t total = (int64_t)(nb - 1) * bs + in_last;
+        n_sel[row] = (int32_t)(total < max_sel ? total : max_sel);
+    }
+}
+
+}  // namespace
+
+int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0, int index_heads,
+                     int index_dim, int block, int keep_blocks, float *scores, int64_t score_stride,
+                     int32_t *blk_out, int32_t *sel, int64_t max_sel, int32_t *n_sel, hipStream_t s) {
+    CWICK_REQUIRE(idx_keys && iq && scores && sel, "mm_select: null pointer");
+    CWICK_REQUIRE(batch >= 1 && batch <= 65535 && limit0 >= 1 && limit0 + batch - 1 <= ((int64_t)1 << 30),
+                  "mm_select: batch %d, first limit %lld", batch, (long long)limit0);
+    CWICK_REQUIRE(index_heads >= 1 && index_heads <= MM_MAX_HEADS && index_dim >= 8 && index_dim <= MM_MAX_DIM &&
+                      index_dim % 8 == 0,
+                  "mm_select: %d index heads of %d dims (1..%d heads, dims a multiple of 8 up to %d)", index_heads,
+                  index_dim, MM_MAX_HEADS, MM_MAX_DIM);
+    CWICK_REQUIRE(block >= 1 && keep_blocks >= 1 && keep_blocks <= 4096, "mm_select: block %d, blocks kept %d", block,
+                  keep_blocks);
+    const int64_t limit_max = limit0 + batch - 1;
+    CWICK_REQUIRE(score_stride >= limit_max, "mm_select: score rows of %lld hold fewer than %lld positions",
+                  (long long)score_stride, (long long)limit_max);
+    CWICK_REQUIRE(max_sel >= 1 && max_sel <= ((int64_t)1 << 24), "mm_select: max_sel %lld", (long long)max_sel);
+    CWICK_REQUIRE(((uintptr_t)idx_keys) % 16 == 0, "mm_select: index keys must be 16-byte aligned");
+    const int64_t nblk_max = (limit_max + block - 1) / block;
+    // rows this short are selected by the one-workgroup top-k kernels, which take no workspace:
+    // the block scores can sit in this call's
+    CWICK_REQUIRE(nblk_max < 16384, "mm_select: %lld blocks (at most 16383)", (long long)nblk_max);
+    const size_t bsc_b = ((size_t)batch * nblk_max * 4 + 255) & ~(size_t)255;
+    char *ws = (char *)workspace(s, bsc_b + (size_t)batch * keep_blocks * 4);
+    CWICK_REQUIRE(ws, "mm_select: workspace allocation failed");
+    float *bsc = (float *)ws;
+    int32_t *blk = (int32_t *)(ws + bsc_b);
+    mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_THREADS - 1) / MM_THREADS), batch), MM_THREADS, 0, s>>>(
+        idx_keys, iq, limit0, index_heads, index_dim, scores, score_stride);
+    mm_blockmax_kernel<<<dim3((unsigned)((nblk_max + 3) / 4), batch), MM_THREADS, 0, s>>>(scores, score_stride, limit0,
+                                                                                      block, nblk_max, bsc);
+    CWICK_HIP_CALL(hipGetLastError());
+    if (!launch_topk(bsc, batch, nblk_max, keep_blocks, blk, s)) return 0;
+    mm_expand_kernel<<<dim3(batch), MM_THREADS, 0, s>>>(blk, keep_blocks, limit0, block, blk_out, sel, max_sel, n_sel);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
+}  // namespace cwick

@@ -1096,6 +1096,15 @@ int cwick_hip_candidate_apply_dev(float *scores, const uint8_t *cand, int batch,
     return launch_candidate_apply(scores, cand, batch, n, (hipStream_t)stream);
 }
 
+int cwick_hip_mm_select_dev(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0, int index_heads,
+                            int index_dim, int block, int keep_blocks, float *scores, int64_t score_stride,
+                            int32_t *blk_out, int32_t *sel, int64_t max_sel, int32_t *n_sel, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_mm_select(idx_keys, iq, batch, limit0, index_heads, index_dim, block, keep_blocks, scores,
+                            score_stride, blk_out, sel, max_sel, n_sel, (hipStream_t)stream);
+}
+
 int cwick_hip_latent_read_f32(cwick_hip_latent *c, int slot, int64_t pos0, int64_t n, float *rows) {
     clear_error();
     LATENT_RANGE_CHECK("latent_read_f32");

@@ -94,6 +94,7 @@ SIGNATURES = {
     "cwick_hip_ikeys_pool_append_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _flt, _int, _vp, _vp]),
     "cwick_hip_candidate_select_dev": (_int, [_vp, _int, _i64, _int, _i64, _vp, _vp]),
     "cwick_hip_candidate_apply_dev": (_int, [_vp, _vp, _int, _i64, _vp]),
+    "cwick_hip_mm_select_dev": (_int, [_vp, _vp, _int, _i64, _int, _int, _int, _int, _vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "cwick_hip_latent_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
     "cwick_hip_ikeys_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
     "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
@@ -562,6 +563,14 @@ def gqa_prepare_dev(q_proj, q_head_stride, k_proj, v_proj, n, pos0, n_heads, n_k
 def candidate_select_dev(scores, batch, n, block, keep_blocks, cand, stream=None, raw=False):
     rc = lib().cwick_hip_candidate_select_dev(_dp(scores), batch, n, block, keep_blocks, _dp(cand), stream)
     return rc if raw else _check(rc, "candidate_select_dev")
+
+
+def mm_select_dev(idx_keys, iq, batch, limit0, index_heads, index_dim, block, keep_blocks, scores, score_stride,
+                  blk_out, sel, max_sel, n_sel, stream=None, raw=False):
+    rc = lib().cwick_hip_mm_select_dev(_dp(idx_keys), _dp(iq), batch, limit0, index_heads, index_dim, block,
+                                       keep_blocks, _dp(scores), score_stride, _dp(blk_out), _dp(sel), max_sel,
+                                       _dp(n_sel), stream)
+    return rc if raw else _check(rc, "mm_select_dev")
 
 
 def candidate_apply_dev(scores, cand, batch, n, stream=None):

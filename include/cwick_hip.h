@@ -370,9 +370,8 @@ int cwick_hip_gqa_prepare_dev(const float *q_proj, int64_t q_head_stride, const 
 /* Replaces the attention of the block-sparse GQA decode (src/mm_model.c:
  * 1962-2047: per head, scores over the selected positions selpos[] with the
  * kv head h / group, max, exp, sum, normalise, weighted sum of the V rows).
- * sel[i] is a cache row; the caller expands its selected blocks
- * (mm_select_blocks, :1733-1761) into positions as the reference does
- * (:1966-1973).  Entries that are negative or not below the number of rows
+ * sel[i] is a cache row; cwick_hip_mm_select_dev below writes the list on
+ * the device.  Query heads per kv head: 1, 2, 4, 8 or 16.  Entries that are negative or not below the number of rows
  * carry no weight; a list without a valid entry gives zeros.  Softmax is a sum:
  * the order of the list does not matter beyond rounding. */
 int cwick_hip_gqa_decode_sel(cwick_hip_kv *c, const int32_t *sel, int64_t n_list, const uint16_t *q,
@@ -381,6 +380,32 @@ int cwick_hip_gqa_decode_sel_dev(const uint16_t *k, const uint16_t *v, int64_t n
                                  int head_dim, const int32_t *sel, int64_t n_list,
                                  const uint16_t *q, int n_heads, float scale, float *out,
                                  void *stream);
+
+/* Replaces what selects those positions: mm_index_scores (src/mm_model.c:
+ * 1764-1780: per position, the dot of each index head's fp32 query with the
+ * position's bf16 index key, one fused multiply-add per dimension in order
+ * from zero, ReLU, the heads added in head order, no head weights),
+ * mm_select_blocks (:1733-1761: a block scores its largest position score, the
+ * keep_blocks best blocks are kept -- mm_topk, :777-814, whose choice on
+ * tie-free input is the one made here: lowest index first among equal maxima
+ * -- and block limit / block is added when it is not among them, which for a
+ * limit that is a multiple of the block size is a block with nothing written
+ * yet) and the loop that writes the kept blocks out as positions (:1969-1976).
+ * Query t of the batch stands at position limit0 - 1 + t and sees limit0 + t
+ * positions, as the queries of a prefill chunk do (:1962-1967); a decode step
+ * is batch 1.  idx_keys bf16 [limit0 + batch - 1][index_dim] (one layer's slice
+ * of the reference's idxcache), iq fp32 [batch][index_heads][index_dim],
+ * scores fp32 [batch][score_stride] (out; row t is filled up to its limit),
+ * blk_out int32 [batch][keep_blocks + 1] (out, may be NULL; ascending, -1
+ * padded), sel int32 [batch][max_sel] (out; the positions in the reference's
+ * order, cut at max_sel as the reference cuts at 4096, then -1: what
+ * cwick_hip_gqa_decode_sel_dev takes with n_list = max_sel), n_sel int32
+ * [batch] (out, may be NULL).  1..8 index heads, index_dim a multiple of 8 up
+ * to 512, at most 16383 blocks. */
+int cwick_hip_mm_select_dev(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0,
+                            int index_heads, int index_dim, int block, int keep_blocks,
+                            float *scores, int64_t score_stride, int32_t *blk_out,
+                            int32_t *sel, int64_t max_sel, int32_t *n_sel, void *stream);
 
 /* Replaces the closing of an indexer pool (indexer_absorb, src/attention.c:
  * 486-525; the two projections in front of it, :481-482, stay the caller's

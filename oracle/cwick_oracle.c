@@ -63,6 +63,16 @@
  *   orc_candidate_mask / _apply        brute force in numpy, last block always kept, number of
  *                                      blocks kept; the block choice is orc_topk_heap's, which
  *                                      is pinned against oracle/_ref
+ *   orc_mm_index_scores                known answers that separate the fused multiply-add from
+ *                                      multiply-then-add, the serial order from a pairwise one,
+ *                                      ReLU-before-sum and the head order; double brute force:
+ *                                      PARITY UNPINNED against a reference build (the file is
+ *                                      NEON-only, and whether the reference fuses is its
+ *                                      compiler's choice)
+ *   orc_mm_select_blocks               known answers traced by hand through src/mm_model.c:
+ *                                      1733-1761 (newest block present, absent, and not yet
+ *                                      written), brute force in numpy on tie-free scores; the
+ *                                      block choice is orc_topk_heap's, pinned against oracle/_ref
  *   orc_indexer_scores[_ds]            double brute force, ReLU-before-weight, thread
  *                                      count invariance: PARITY UNPINNED against a
  *                                      reference build
@@ -1069,6 +1079,64 @@ ORC_API int orc_candidate_mask(const float *scores, int nvis, int bs, int keep, 
 /* src/ds_model.c:1145-1148: scores outside the candidate blocks become -inf. */
 ORC_API void orc_candidate_apply(float *scores, const uint8_t *cand, int nvis) {
     for (int t = 0; t < nvis; t++) if (!cand[t]) scores[t] = -INFINITY;
+}
+
+/* ------------------------------------------------------------------ */
+/* MiniMax block selection (the second consumer of the gather decode)  */
+/* ------------------------------------------------------------------ */
+
+/* src/mm_model.c:1764-1780 (mm_index_scores): per position the dot of every index head's fp32
+ * query with the position's bf16 index key, accumulated serially from 0 in dimension order,
+ * ReLU, and the heads summed in head order.  No head weights.  The reference writes
+ * `d += qh[i] * k[i]` and leaves contraction to its compiler (clang, which fuses by default);
+ * this file is compiled with contraction off, so the fused form is spelled out. */
+ORC_API void orc_mm_index_scores(const float *iq, const uint16_t *keys, int64_t limit, int ih, int id,
+                                 float *scores) {
+    for (int64_t s = 0; s < limit; s++) {
+        const uint16_t *k = keys + (size_t)s * (size_t)id;
+        float tot = 0.0f;
+        for (int h = 0; h < ih; h++) {
+            const float *qh = iq + (size_t)h * (size_t)id;
+            float d = 0.0f;
+            for (int i = 0; i < id; i++) d = fmaf(qh[i], orc_bf16_to_f32(k[i]), d);
+            if (d > 0.0f) tot += d;
+        }
+        scores[s] = tot;
+    }
+}
+
+/* src/mm_model.c:1733-1761 (mm_select_blocks) and :1969-1976 (the chosen blocks written out as
+ * positions): a block scores the largest position score inside it, the `keep` best blocks are
+ * taken by the heap selector (mm_topk, :777-814, the same sequence of comparisons and swaps as
+ * ds_topk_scores on scores that are not NaN), and block limit / bs is added when it is not among
+ * them -- when limit is a multiple of bs that is a block with no position written yet, which
+ * then contributes no position.  blk_out holds keep + 1 entries; sel holds at most max_sel
+ * positions.  Returns the number of blocks; *n_sel receives the number of positions. */
+ORC_API int orc_mm_select_blocks(const float *scores, int64_t limit, int bs, int keep, int *blk_out,
+                                 int64_t *sel, int64_t max_sel, int64_t *n_sel) {
+    const int64_t nblk = (limit + bs - 1) / bs;
+    float *bsc = malloc(sizeof(float) * (size_t)(nblk + 1));
+    for (int64_t b = 0; b < nblk; b++) {
+        int64_t s0 = b * bs, s1 = s0 + bs;
+        if (s1 > limit) s1 = limit;
+        float best = -1e30f;
+        for (int64_t s = s0; s < s1; s++) best = fmaxf(best, scores[s]);
+        bsc[b] = best;
+    }
+    int nb = orc_topk_heap(bsc, (int)nblk, keep, blk_out);
+    const int newest = (int)(limit / bs);
+    int have = 0;
+    for (int i = 0; i < nb; i++) if (blk_out[i] == newest) have = 1;
+    if (!have) blk_out[nb++] = newest;
+    int64_t ns = 0;
+    for (int b = 0; b < nb && ns < max_sel; b++) {
+        int64_t s0 = (int64_t)blk_out[b] * bs, s1 = s0 + bs;
+        if (s1 > limit) s1 = limit;
+        for (int64_t s = s0; s < s1 && ns < max_sel; s++) sel[ns++] = s;
+    }
+    *n_sel = ns;
+    free(bsc);
+    return nb;
 }
 
 /* ------------------------------------------------------------------ */

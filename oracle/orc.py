@@ -334,6 +334,30 @@ def candidate_apply(scores, cand):
     return sc
 
 
+def mm_index_scores(iq, keys, limit=None):
+    """iq [ih,id] f32, keys [n,id] bf16 bits -> [limit] f32 (src/mm_model.c:1764-1780)."""
+    iq = np.ascontiguousarray(iq, np.float32)
+    keys = np.ascontiguousarray(keys, np.uint16)
+    ih, idim = iq.shape
+    limit = keys.shape[0] if limit is None else int(limit)
+    out = np.empty(limit, np.float32)
+    lib().orc_mm_index_scores(_p(iq, C.c_float), _p(keys, C.c_uint16), C.c_int64(limit), int(ih), int(idim),
+                              _p(out, C.c_float))
+    return out
+
+
+def mm_select_blocks(scores, limit, block, keep, max_sel=4096):
+    """-> (blocks, positions) as src/mm_model.c:1733-1761 and :1969-1976 leave them."""
+    sc = np.ascontiguousarray(scores, np.float32)
+    assert sc.size >= limit
+    blk = np.empty(keep + 1, np.int32)
+    sel = np.empty(max(max_sel, 1), np.int64)
+    ns = C.c_int64(0)
+    nb = lib().orc_mm_select_blocks(_p(sc, C.c_float), C.c_int64(limit), int(block), int(keep), _p(blk, C.c_int32),
+                                    _p(sel, C.c_int64), C.c_int64(max_sel), C.byref(ns))
+    return blk[:nb].copy(), sel[:ns.value].copy()
+
+
 def topk_contract(sc, k):
     sc = np.ascontiguousarray(sc, np.float32)
     out = np.empty(max(min(k, sc.size), 1), np.int32)

@@ -1095,3 +1095,88 @@ def test_gqa_decode_over_selected_blocks(hip, orc, n_rows, nh, nkv, hd, bs, keep
     none = hip.gqa_decode_sel(cache, np.array([-1, -1, n_rows], np.int32), q, c["scale"])
     assert np.all(none == 0.0)
     cache.free()
+
+
+@pytest.mark.parametrize("limit0,batch,ih,idim,bs,keep,max_sel", [
+    (8192, 1, 4, 128, 128, 16, 4096),      # the reference's geometry (src/mm_model.c:1011-1012), a full last block
+    (8000, 1, 4, 128, 128, 16, 4096),      # a partly filled newest block
+    (1020, 8, 4, 128, 128, 3, 4096),       # a chunk whose queries cross a block border (1024)
+    (70, 3, 1, 8, 7, 4, 64),
+    (1, 2, 4, 128, 128, 16, 4096),         # the first positions of a sequence
+    (40000, 2, 8, 64, 64, 20, 1000),       # the list cut at max_sel
+    (300, 1, 2, 512, 128, 16, 4096),       # more blocks asked for than exist
+])
+def test_mm_select_blocks_on_device(hip, orc, limit0, batch, ih, idim, bs, keep, max_sel):
+    """The block selection of the block-sparse decode (src/mm_model.c:1764-1780, :1733-1761,
+    :1969-1976) for a chunk of consecutive queries: position scores bit for bit, the kept blocks
+    and the position list equal to the oracle's."""
+    import torch
+    say("[case] mm select", limit0, batch, ih, idim, bs, keep, max_sel)
+    g = synth.rng(limit0 + 31 * batch + ih)
+    n = limit0 + batch - 1
+    keys = synth.normal_bf16(g, (n, idim))
+    iq = g.standard_normal((batch, ih, idim)).astype(np.float32)
+    stride = n + 5
+    d_keys = torch.from_numpy(keys.view(np.int16)).cuda()
+    d_iq = torch.from_numpy(iq).cuda()
+    d_sc = torch.full((batch, stride), float("nan"), dtype=torch.float32, device="cuda")
+    d_blk = torch.full((batch, keep + 1), 77, dtype=torch.int32, device="cuda")
+    d_sel = torch.full((batch, max_sel), 77, dtype=torch.int32, device="cuda")
+    d_ns = torch.full((batch,), 77, dtype=torch.int32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.mm_select_dev(d_keys, d_iq, batch, limit0, ih, idim, bs, keep, d_sc, stride, d_blk, d_sel, max_sel, d_ns, s)
+    torch.cuda.synchronize()
+    sc, blk, sel, ns = d_sc.cpu().numpy(), d_blk.cpu().numpy(), d_sel.cpu().numpy(), d_ns.cpu().numpy()
+    for t in range(batch):
+        limit = limit0 + t
+        ref_sc = orc.mm_index_scores(iq[t], keys, limit)
+        assert np.array_equal(sc[t, :limit].view(np.uint32), ref_sc.view(np.uint32)), "query %d: scores differ" % t
+        assert np.isnan(sc[t, limit:]).all(), "query %d: scores written past the limit" % t
+        rblk, rpos = orc.mm_select_blocks(ref_sc, limit, bs, keep, max_sel)
+        assert list(blk[t, :rblk.size]) == list(rblk) and (blk[t, rblk.size:] == -1).all(), "query %d: blocks" % t
+        assert ns[t] == rpos.size
+        assert list(sel[t, :rpos.size]) == list(rpos) and (sel[t, rpos.size:] == -1).all(), "query %d: positions" % t
+    # blk_out and n_sel may be left out
+    d_sel2 = torch.full((batch, max_sel), 77, dtype=torch.int32, device="cuda")
+    hip.mm_select_dev(d_keys, d_iq, batch, limit0, ih, idim, bs, keep, d_sc, stride, None, d_sel2, max_sel, None, s)
+    torch.cuda.synchronize()
+    assert torch.equal(d_sel, d_sel2)
+    rc = hip.mm_select_dev(d_keys, d_iq, batch, limit0, 9, idim, bs, keep, d_sc, stride, None, d_sel2, max_sel, None, s,
+                           raw=True)
+    assert rc == 0 and "index heads" in hip.last_error()
+
+
+@pytest.mark.parametrize("n_rows,nh,nkv,hd", [(5000, 64, 4, 128), (2304, 32, 2, 256)])
+def test_mm_block_sparse_decode_chain(hip, orc, n_rows, nh, nkv, hd):
+    """Selection and attention of the block-sparse decode chained on the device with nothing
+    crossing to the host in between, sixteen query heads per kv head (the reference's 64/4,
+    src/mm_model.c:1962-2047): against the oracle's selection and its decode over the gathered rows."""
+    import torch
+    say("[case] mm chain", n_rows, nh, nkv, hd)
+    g = synth.rng(4100 + n_rows)
+    ih, idim, bs, keep = 4, 128, 128, 16
+    c = synth.cfg1_gqa_decode(n_rows, nh, nkv, hd, seed=4200 + n_rows)
+    keys = synth.normal_bf16(g, (n_rows, idim))
+    iq = g.standard_normal((1, ih, idim)).astype(np.float32)
+    cache = hip.KVCache(n_rows, nkv, hd)
+    cache.write(0, c["k"].reshape(n_rows, -1), c["v"].reshape(n_rows, -1))
+    max_sel = (keep + 1) * bs
+    d_keys = torch.from_numpy(keys.view(np.int16)).cuda()
+    d_iq = torch.from_numpy(iq).cuda()
+    d_sc = torch.empty((1, n_rows), dtype=torch.float32, device="cuda")
+    d_sel = torch.empty((1, max_sel), dtype=torch.int32, device="cuda")
+    d_q = torch.from_numpy(c["q"].view(np.int16)).cuda()
+    d_out = torch.empty((nh, hd), dtype=torch.float32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.mm_select_dev(d_keys, d_iq, 1, n_rows, ih, idim, bs, keep, d_sc, n_rows, None, d_sel, max_sel, None, s)
+    hip.gqa_decode_sel_dev(cache.k_dev(), cache.v_dev(), n_rows, nkv, hd, d_sel, max_sel, d_q, nh, c["scale"], d_out, s)
+    torch.cuda.synchronize()
+    _, rpos = orc.mm_select_blocks(orc.mm_index_scores(iq[0], keys), n_rows, bs, keep, max_sel)
+    sel = d_sel.cpu().numpy()[0]
+    assert list(sel[:rpos.size]) == list(rpos)
+    ref = orc.gqa_decode(c["q"], c["k"][rpos], c["v"][rpos], c["scale"])
+    assert_close(d_out.cpu().numpy(), ref, "mm chain %d rows, %d positions, %d/%d heads" % (n_rows, rpos.size, nh, nkv))
+    # the dense decode with sixteen heads per kv head
+    dense = hip.gqa_decode(cache, n_rows, c["q"], c["scale"])
+    assert_close(dense, orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"], nthreads=0), "gqa decode group 16")
+    cache.free()

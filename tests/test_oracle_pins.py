@@ -284,3 +284,87 @@ def test_dot_f32_order(orc):
     g = synth.rng(6)
     x, y = g.standard_normal(576).astype(np.float32), g.standard_normal(576).astype(np.float32)
     assert abs(orc.dot_f32(x, y) - float(x.astype(np.float64) @ y.astype(np.float64))) < 1e-3
+
+
+# ------------------------------------------------------------------ MiniMax block selection
+def _bf16(x):
+    return synth.f32_to_bf16(np.asarray(x, np.float32))
+
+
+def test_mm_index_scores_known_answers(orc):
+    """src/mm_model.c:1764-1780.  Each case fails for one plausible mistake."""
+    one = _bf16([1.0])[0]
+    # fused multiply-add: the low bit of the second product survives only when it is not rounded
+    # before the addition (multiply-then-add gives 0)
+    q = np.array([[-(1.0 + 2.0 ** -7 + 2.0 ** -23), 1.0 + 2.0 ** -23]], np.float32)
+    k = np.array([[one, _bf16([1.0 + 2.0 ** -7])[0]]], np.uint16)
+    assert orc.mm_index_scores(q, k)[0] == np.float32(2.0 ** -30)
+    # serial order from zero: 2^24 + 1 + 1 stays 2^24, then -2^24 + 4 leaves 4 (pairwise 5, exact 6)
+    q = np.array([[2.0 ** 24, 1.0, 1.0, -(2.0 ** 24) + 4.0]], np.float32)
+    k = np.full((1, 4), one, np.uint16)
+    assert orc.mm_index_scores(q, k)[0] == np.float32(4.0)
+    # ReLU per head before the sum, heads added in head order, no weights
+    q = np.array([[2.0 ** 24], [-5.0], [1.0]], np.float32)
+    k = np.array([[one]], np.uint16)
+    assert orc.mm_index_scores(q, k)[0] == np.float32(2.0 ** 24)
+    q = np.array([[1.0], [1.0], [2.0 ** 24]], np.float32)
+    assert orc.mm_index_scores(q, k)[0] == np.float32(2.0 ** 24 + 2.0)
+    # the key is bf16 bits widened by a shift; a negative dot scores zero
+    k = np.array([[0xC000], [0x3F80], [0x4040]], np.uint16)             # -2, 1, 3
+    q = np.array([[1.5]], np.float32)
+    assert list(orc.mm_index_scores(q, k)) == [0.0, 1.5, 4.5]
+    # only the first `limit` positions are scored
+    assert orc.mm_index_scores(q, k, limit=2).shape == (2,)
+
+
+def test_mm_index_scores_vs_double(orc):
+    g = synth.rng(81)
+    for n, ih, idim in [(300, 4, 128), (17, 1, 8), (64, 8, 64)]:
+        q = g.standard_normal((ih, idim)).astype(np.float32)
+        kb = synth.normal_bf16(g, (n, idim))
+        kf = synth.bf16_to_f32(kb).astype(np.float64)
+        want = np.maximum(kf @ q.astype(np.float64).T, 0.0).sum(axis=1)
+        got = orc.mm_index_scores(q, kb)
+        assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+
+
+def test_mm_select_blocks_known_answers(orc):
+    """Traced by hand through src/mm_model.c:1733-1761 and :1969-1976 (block size 4)."""
+    a = np.array([0.1, 0.9, 0.2, 0.3, 0.5, 0.4, 0.6, 0.2, 0.05, 0.07], np.float32)
+    # block maxima 0.9, 0.6, 0.07; two kept: 0 and 1; the newest block, 10 / 4 = 2, is added
+    blk, pos = orc.mm_select_blocks(a, 10, 4, 2)
+    assert list(blk) == [0, 1, 2] and list(pos) == list(range(10))
+    # a limit that is a multiple of the block size: the added block is 8 / 4 = 2, which holds no
+    # written position, so the list is block 0 alone (positions 4..7 are NOT attended)
+    blk, pos = orc.mm_select_blocks(a, 8, 4, 1)
+    assert list(blk) == [0, 2] and list(pos) == [0, 1, 2, 3]
+    # the newest block already among the kept ones: nothing is added
+    b = a.copy(); b[8] = 5.0
+    blk, pos = orc.mm_select_blocks(b, 10, 4, 2)
+    assert list(blk) == [0, 2] and list(pos) == [0, 1, 2, 3, 8, 9]
+    # at most max_sel positions, cut in block order
+    blk, pos = orc.mm_select_blocks(a, 10, 4, 2, max_sel=6)
+    assert list(blk) == [0, 1, 2] and list(pos) == [0, 1, 2, 3, 4, 5]
+    # more blocks asked for than exist
+    blk, pos = orc.mm_select_blocks(a, 10, 4, 5)
+    assert list(blk) == [0, 1, 2] and list(pos) == list(range(10))
+    # a single position
+    blk, pos = orc.mm_select_blocks(a, 1, 4, 2)
+    assert list(blk) == [0] and list(pos) == [0]
+    # scores past the limit are not read: block 1's 0.6 at position 6 is outside limit 6
+    blk, pos = orc.mm_select_blocks(a, 6, 4, 1)
+    assert list(blk) == [0, 1] and list(pos) == [0, 1, 2, 3, 4, 5]
+
+
+def test_mm_select_blocks_vs_brute_force(orc):
+    g = synth.rng(82)
+    for limit, bs, keep in [(1000, 128, 3), (4096, 128, 16), (4097, 128, 16), (70, 7, 4), (129, 128, 16), (5000, 64, 20)]:
+        sc = np.abs(g.standard_normal(limit)).astype(np.float32)
+        nblk = -(-limit // bs)
+        bmax = np.array([sc[b * bs:min((b + 1) * bs, limit)].max() for b in range(nblk)])
+        assert len(set(bmax.tolist())) == nblk                          # tie-free
+        want = set(np.argsort(-bmax, kind="stable")[:keep].tolist()) | {limit // bs}
+        blk, pos = orc.mm_select_blocks(sc, limit, bs, keep, max_sel=1 << 20)
+        assert list(blk) == sorted(want)
+        wpos = [s for b in sorted(want) for s in range(b * bs, min((b + 1) * bs, limit))]
+        assert list(pos) == wpos
