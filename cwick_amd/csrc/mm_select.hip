@@ -8,8 +8,9 @@
 //   1. mm_index_scores_kernel   one thread per position: for every index head the dot of the
 //      head's fp32 query with the position's bf16 key, a fused multiply-add per dimension in
 //      dimension order from zero (the reference's serial loop), ReLU, the heads added in head
-//      order.  The query sits in LDS and is read as a broadcast; a thread streams its own
-//      256-byte key row in 16-byte pieces.
+//      order.  The query is read through the scalar unit; a thread requests its whole
+//      256-byte key row in 16-byte pieces before it uses the first (the serial order ties a key
+//      to one thread, so the row cannot be spread over lanes).
 //   2. mm_blockmax_kernel       one wave per block: the largest score inside the block, started
 //      from -1e30 like the reference; blocks past a query's last one get -inf so that rows of
 //      a chunk with different block counts share one top-k launch.
@@ -26,45 +27,55 @@ namespace cwick {
 namespace {
 
 constexpr int MM_THREADS = 256;
+constexpr int MM_SCORE_THREADS = 64;        // one wave: a short context still spreads over many CUs
 constexpr int MM_MAX_HEADS = 8;
 constexpr int MM_MAX_DIM = 512;
 
-__global__ void __launch_bounds__(MM_THREADS)
+__global__ void __launch_bounds__(MM_SCORE_THREADS)
 mm_index_scores_kernel(const uint16_t *__restrict__ keys, const float *__restrict__ iq, int64_t limit0, int ih, int id,
                        float *__restrict__ scores, int64_t score_stride) {
-    __shared__ __attribute__((aligned(16))) float qs[MM_MAX_HEADS * MM_MAX_DIM];
     const int row = blockIdx.y;
     const int64_t limit = limit0 + row;
-    if ((int64_t)blockIdx.x * MM_THREADS >= limit) return;          // the whole workgroup: before any barrier
-    const float *q = iq + (size_t)row * ih * id;
-    for (int i = threadIdx.x; i < ih * id; i += MM_THREADS) qs[i] = q[i];
-    __syncthreads();
-    const int64_t s = (int64_t)blockIdx.x * MM_THREADS + threadIdx.x;
+    if ((int64_t)blockIdx.x * MM_SCORE_THREADS >= limit) return;
+    const int64_t s = (int64_t)blockIdx.x * MM_SCORE_THREADS + threadIdx.x;
     const int64_t sc = s < limit ? s : limit - 1;                   // threads past the end read the last row
     const u32x4 *kp = (const u32x4 *)(keys + (size_t)sc * id);
+    const int chunks = id / 8;
+    // sixteen pieces of the row (a whole 128-dimension key) are requested before the first is
+    // used: one round trip to memory per key
+    constexpr int G = 16;
+    u32x4 kw[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) kw[g] = kp[g < chunks ? g : chunks - 1];
+    // the query is the same for every thread: its address is uniform, so it arrives through the
+    // scalar unit, eight values a load, and enters the multiply-adds as a scalar operand
+    const float *__restrict__ q = iq + (size_t)row * ih * id;
     float d[MM_MAX_HEADS];
 #pragma unroll
     for (int h = 0; h < MM_MAX_HEADS; h++) d[h] = 0.0f;
-    const int chunks = id / 8;
-    u32x4 kw = kp[0];
-    for (int c = 0; c < chunks; c++) {
-        const u32x4 cur = kw;
-        if (c + 1 < chunks) kw = kp[c + 1];
-        float kf[8];
+    for (int c0 = 0; c0 < chunks; c0 += G) {
+        if (c0) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            kf[2 * i] = bf16lo_to_f32(cur[i]);
-            kf[2 * i + 1] = bf16hi_to_f32(cur[i]);
+            for (int g = 0; g < G; g++) kw[g] = kp[c0 + g < chunks ? c0 + g : chunks - 1];
         }
 #pragma unroll
-        for (int h = 0; h < MM_MAX_HEADS; h++) {
-            if (h < ih) {                                           // uniform
-                const f32x4 qa = *(const f32x4 *)(qs + h * id + c * 8);
-                const f32x4 qb = *(const f32x4 *)(qs + h * id + c * 8 + 4);
+        for (int g = 0; g < G; g++) {
+            if (c0 + g < chunks) {                                  // uniform
+                const int c = c0 + g;
+                float kf[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) d[h] = __builtin_fmaf(qa[i], kf[i], d[h]);
+                for (int i = 0; i < 4; i++) {
+                    kf[2 * i] = bf16lo_to_f32(kw[g][i]);
+                    kf[2 * i + 1] = bf16hi_to_f32(kw[g][i]);
+                }
 #pragma unroll
-                for (int i = 0; i < 4; i++) d[h] = __builtin_fmaf(qb[i], kf[4 + i], d[h]);
+                for (int h = 0; h < MM_MAX_HEADS; h++) {
+                    if (h < ih) {                                   // uniform
+                        const float *qh = q + h * id + c * 8;
+#pragma unroll
+                        for (int i = 0; i < 8; i++) d[h] = __builtin_fmaf(qh[i], kf[i], d[h]);
+                    }
+                }
             }
         }
     }
@@ -166,7 +177,8 @@ int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64
     CWICK_REQUIRE(ws, "mm_select: workspace allocation failed");
     float *bsc = (float *)ws;
     int32_t *blk = (int32_t *)(ws + bsc_b);
-    mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_THREADS - 1) / MM_THREADS), batch), MM_THREADS, 0, s>>>(
+    mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS), batch),
+                             MM_SCORE_THREADS, 0, s>>>(
         idx_keys, iq, limit0, index_heads, index_dim, scores, score_stride);
     mm_blockmax_kernel<<<dim3((unsigned)((nblk_max + 3) / 4), batch), MM_THREADS, 0, s>>>(scores, score_stride, limit0,
                                                                                       block, nblk_max, bsc);

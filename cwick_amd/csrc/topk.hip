@@ -156,8 +156,9 @@ topk_radix_kernel(const float *__restrict__ scores, int64_t n, int64_t k, int32_
 // Wave w owns the consecutive elements [w * 64 * ept, (w + 1) * 64 * ept); inside it lane l
 // holds elements base + 64 j + l, so the loads are coalesced and index order is (j, lane):
 // positions inside a wave come from ballots, positions of the waves from one block scan.
-constexpr int TOPK_EPT = 64;                   // keys per thread
+constexpr int TOPK_EPT = 64;                   // keys per thread at most; shorter rows take a kernel unrolled for fewer
 
+template <int EPT>
 __global__ void __launch_bounds__(TOPK_THREADS)
 topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
                       int32_t *__restrict__ out) {
@@ -174,14 +175,14 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     const int64_t kk = k < n ? k : n;
     for (int64_t i = kk + tid; i < k; i += TOPK_THREADS) dst[i] = -1;
 
-    const int ept = (int)((n + TOPK_THREADS - 1) / TOPK_THREADS);     // <= 64
+    const int ept = (int)((n + TOPK_THREADS - 1) / TOPK_THREADS);     // <= EPT
     const int64_t wbase = (int64_t)wave * 64 * ept;
     // this lane holds elements j < jv
     int64_t left = n - wbase - lane;
     const int jv = left <= 0 ? 0 : (int)((left + 63) / 64 < ept ? (left + 63) / 64 : ept);
-    uint32_t key[TOPK_EPT];
+    uint32_t key[EPT];
 #pragma unroll
-    for (int j = 0; j < TOPK_EPT; j++) key[j] = j < jv ? topk_key(sc[wbase + 64 * j + lane]) : 0u;
+    for (int j = 0; j < EPT; j++) key[j] = j < jv ? topk_key(sc[wbase + 64 * j + lane]) : 0u;
     if (tid == 0) {
         sh_prefix = 0u;
         sh_remaining = (uint32_t)kk;
@@ -197,7 +198,7 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
         __syncthreads();
         if (shift == 24) {
 #pragma unroll
-            for (int j = 0; j < TOPK_EPT; j++)
+            for (int j = 0; j < EPT; j++)
                 if (j < jv) atomicAdd(&hist32[(key[j] >> 24) * 32 + (lane & 31)], 1u);
             __syncthreads();
             if (tid < 256) {
@@ -208,7 +209,7 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < TOPK_EPT; j++)
+            for (int j = 0; j < EPT; j++)
                 if (j < jv && (key[j] & mask) == prefix) atomicAdd(&hist[(key[j] >> shift) & 0xFFu], 1u);
         }
         __syncthreads();
@@ -243,7 +244,7 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     // ---- 2. ordered emit ----
     uint32_t w_gt = 0u, w_eq = 0u;         // wave totals (uniform)
 #pragma unroll
-    for (int j = 0; j < TOPK_EPT; j++) {
+    for (int j = 0; j < EPT; j++) {
         w_gt += (uint32_t)__builtin_popcountll(__ballot(j < jv && key[j] > T));
         w_eq += (uint32_t)__builtin_popcountll(__ballot(j < jv && key[j] == T));
     }
@@ -261,7 +262,7 @@ topk_radix_reg_kernel(const float *__restrict__ scores, int64_t n, int64_t k,
     }
     const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
 #pragma unroll
-    for (int j = 0; j < TOPK_EPT; j++) {
+    for (int j = 0; j < EPT; j++) {
         const bool gt = j < jv && key[j] > T;
         const bool eq = j < jv && key[j] == T;
         const uint64_t m_eq = __ballot(eq);
@@ -865,8 +866,14 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     }
     {
         ProfScope ps(CWICK_HIP_PROF_TOPK, s);
-        if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)
-            topk_radix_reg_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        if (n <= (int64_t)TOPK_THREADS)
+            topk_radix_reg_kernel<1><<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        else if (n <= (int64_t)TOPK_THREADS * 4)
+            topk_radix_reg_kernel<4><<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        else if (n <= (int64_t)TOPK_THREADS * 16)
+            topk_radix_reg_kernel<16><<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
+        else if (n <= (int64_t)TOPK_THREADS * TOPK_EPT)
+            topk_radix_reg_kernel<TOPK_EPT><<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
         else
             topk_radix_kernel<<<batch, TOPK_THREADS, 0, s>>>(scores, n, k, out_idx);
     }
