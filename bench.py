@@ -345,6 +345,59 @@ def bench_cfg5(hip, synth, orc, T, stream, a, shared=False):
 
 
 # ---------------------------------------------------------------- CPU baseline (oracle, "port")
+def bench_cfg6(hip, synth, orc, T, stream, a):
+    """Not one of the five configurations the metric names: the block-sparse GQA decode
+    (src/mm_model.c:1962-2047 with its block selection, :1733-1780) at the reference's geometry,
+    timed so that the kernels of that path have a committed command to profile."""
+    import torch
+    n, nh, nkv, hd, ih, idim, bs, keep = 65536, 64, 4, 128, 4, 128, 128, 16
+    g = synth.rng(synth.SEED0 + 6)
+    c = synth.cfg1_gqa_decode(n, nh, nkv, hd, seed=synth.SEED0 + 6)
+    keys_h = synth.normal_bf16(g, (n, idim))
+    iq_h = g.standard_normal((1, ih, idim)).astype(np.float32)
+    k, v, q, keys, iq = dev(c["k"]), dev(c["v"]), dev(c["q"]), dev(keys_h), dev(iq_h)
+    max_sel = (keep + 1) * bs
+    sc = torch.empty((1, n), dtype=torch.float32, device="cuda")
+    sel = torch.empty((1, max_sel), dtype=torch.int32, device="cuda")
+    out = torch.empty((nh, hd), dtype=torch.float32, device="cuda")
+
+    def step():
+        hip.mm_select_dev(keys, iq, 1, n, ih, idim, bs, keep, sc, n, None, sel, max_sel, None, stream)
+        hip.gqa_decode_sel_dev(k, v, n, nkv, hd, sel, max_sel, q, nh, c["scale"], out, stream)
+    wall, kern, spread = T.run(step)
+    # the selection reads every index key once; the attention reads the listed K and V rows
+    alg_sel = n * idim * 2 + n * 4
+    alg_att = 2 * max_sel * nkv * hd * 2
+    ms = kern["mm select kernels"]
+    t_sel = ms["avg_us"] * ms["launches"] / T.steps * 1e-6             # two timed sections per call
+    r = {"workload": "block-sparse GQA decode 64q/4kv/hd128: 4x128 index scores over 65536 bf16 keys -> 16 of 512 "
+                     "blocks + the newest -> attention over 2176 positions (outside BASELINE's five configurations)",
+         "us_per_step": wall * 1e6, "step_us": spread, "kernels": kern,
+         "alg_bytes_select": alg_sel, "alg_bytes_attention": alg_att,
+         "roofline": roofline("hbm", alg_sel, t_sel, HBM_PEAK_GBS, "GB/s", measured=CEIL.get("hbm_GBps"))}
+    if orc:
+        _, rpos = orc.mm_select_blocks(orc.mm_index_scores(iq_h[0], keys_h), n, bs, keep, max_sel)
+        got_sel = sel.cpu().numpy()[0]
+        same = bool(np.array_equal(got_sel[:rpos.size], rpos) and (got_sel[rpos.size:] == -1).all())
+        ref = orc.gqa_decode(c["q"], c["k"][rpos], c["v"][rpos], c["scale"], nthreads=0)
+        ok, d = close(out.cpu().numpy(), ref)
+        r["checked"], r["check_maxabs"] = bool(same and ok), d
+        r["check"] = "the position list bit for bit, the output against the oracle's decode over the listed rows"
+        if not a.no_cpu:
+            th = cpu_threads(orc)
+
+            def cpu_step():
+                s_ = orc.mm_index_scores(iq_h[0], keys_h)
+                _, pos = orc.mm_select_blocks(s_, n, bs, keep, max_sel)
+                orc.gqa_decode(c["q"], c["k"][pos], c["v"][pos], c["scale"], 16, th)
+            mean, best, reps = timed(orc, cpu_step, 2.0, 2)
+            r["cpu_baseline"] = {"value": round(mean * 1e6, 1), "unit": "us/token", "cores": th, "kind": "port",
+                                 "sample": "%d full steps (mean; best %.0f us): serial index scores on one thread "
+                                           "(src/mm_model.c:1764-1780), block selection, attention over the listed rows"
+                                           % (reps, best * 1e6)}
+    return r
+
+
 def cpu_baseline_cfg3(orc, c, budget_s):
     """The oracle's restatement of src/attention.c:749-811 over BASELINE's FP8 storage, all
     host cores, bounded to about `budget_s` seconds of work."""
@@ -364,7 +417,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--configs", default="1,2,3,4,5",
-                    help="which configurations to time besides the headline (3 always runs)")
+                    help="which configurations to time besides the headline (3 always runs); 6 is the "
+                         "block-sparse GQA decode, which the metric does not name")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-check", action="store_true", help="skip the output checks (and the CPU baselines)")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the read and matrix-core probes")
@@ -427,7 +481,8 @@ def main():
     # enough steps that the fixed cost of the two device syncs around the timed region (0.1 to 1 ms
     # on this stack, whatever is enqueued) stays below a per cent of the region
     side = {1: (bench_cfg1, a.steps), 2: (bench_cfg2, max(20, a.steps // 4)),
-            4: (bench_cfg4, max(2, a.steps // 50)), 5: (bench_cfg5, max(3, a.steps // 2))}
+            4: (bench_cfg4, max(2, a.steps // 50)), 5: (bench_cfg5, max(3, a.steps // 2)),
+            6: (bench_cfg6, max(3, a.steps // 2))}
     for i in sorted(wanted - {3}):
         fn, k = side[i]
         Ti = Timer(hip, torch, k, max(1, min(a.warmup, k // 2)))

@@ -177,14 +177,20 @@ int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64
     CWICK_REQUIRE(ws, "mm_select: workspace allocation failed");
     float *bsc = (float *)ws;
     int32_t *blk = (int32_t *)(ws + bsc_b);
-    mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS), batch),
-                             MM_SCORE_THREADS, 0, s>>>(
-        idx_keys, iq, limit0, index_heads, index_dim, scores, score_stride);
-    mm_blockmax_kernel<<<dim3((unsigned)((nblk_max + 3) / 4), batch), MM_THREADS, 0, s>>>(scores, score_stride, limit0,
-                                                                                      block, nblk_max, bsc);
+    {
+        ProfScope ps(CWICK_HIP_PROF_MM_SELECT, s);
+        mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS), batch),
+                                 MM_SCORE_THREADS, 0, s>>>(idx_keys, iq, limit0, index_heads, index_dim, scores,
+                                                            score_stride);
+        mm_blockmax_kernel<<<dim3((unsigned)((nblk_max + 3) / 4), batch), MM_THREADS, 0, s>>>(scores, score_stride,
+                                                                                          limit0, block, nblk_max, bsc);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     if (!launch_topk(bsc, batch, nblk_max, keep_blocks, blk, s)) return 0;
-    mm_expand_kernel<<<dim3(batch), MM_THREADS, 0, s>>>(blk, keep_blocks, limit0, block, blk_out, sel, max_sel, n_sel);
+    {
+        ProfScope ps(CWICK_HIP_PROF_MM_SELECT, s);
+        mm_expand_kernel<<<dim3(batch), MM_THREADS, 0, s>>>(blk, keep_blocks, limit0, block, blk_out, sel, max_sel, n_sel);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -1034,7 +1034,8 @@ int cwick_hip_prof_read(int which, double *total_ms, int64_t *launches) {
 const char *cwick_hip_prof_name(int which) {
     static const char *names[CWICK_HIP_PROF_COUNT] = {
         "gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel"};
+        "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel",
+        "mm select kernels"};
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 

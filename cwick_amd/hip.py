@@ -580,7 +580,8 @@ def candidate_apply_dev(scores, cand, batch, n, stream=None):
 
 # ------------------------------------------------------------------ phase timers
 PROF_NAMES = ["gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
-              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel"]
+              "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel",
+              "mm select kernels"]
 
 
 def prof_enable(on=True):
