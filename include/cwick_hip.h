@@ -142,7 +142,7 @@ float *cwick_hip_ikeys_scales_dev(cwick_hip_ikeys *c, int slot);
  * dec_out_slices (src/q35_model.c:1656-1701).  One query position, every
  * head: out[h] = softmax_t(scale * q[h].K[t][h/group]) . V[.][h/group] over
  * t in [0, n_keys).  q [n_heads][head_dim] bf16, out [n_heads][head_dim] fp32.
- * Supported: head_dim 256 or 128, group = n_heads/n_kv_heads in {1,2,4,8},
+ * Supported: head_dim 256 or 128, group = n_heads/n_kv_heads in {1,2,4,8,16},
  * 1 <= n_keys <= capacity. */
 int cwick_hip_gqa_decode(cwick_hip_kv *c, int64_t n_keys, const uint16_t *q,
                          int n_heads, float scale, float *out);
