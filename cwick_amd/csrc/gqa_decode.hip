@@ -241,15 +241,17 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     const int n_heads = n_units * GROUP;
     constexpr int LPK = HD / 8, NGRP = GQA_DEC_THREADS / LPK;
     constexpr int step = NGRP * GQA_DEC_KB;   // rows one workgroup consumes per iteration
-    // enough workgroups for ~2 per CU, each at least one full step
+    // About one workgroup per CU, each with whole steps: a slice is the share of a workgroup
+    // rounded DOWN to whole steps (a few workgroups more than CUs are cheaper than workgroups
+    // half as many and twice as long; twice as many with one step each cost a microsecond in
+    // partials written and merged).  4096 keys on 4 kv heads: 64 slices of two steps.
     const char *env = getenv("CWICK_HIP_GQA_WG_PER_CU");
-    int per_cu = env ? atoi(env) : 2;
-    if (per_cu < 1 || per_cu > 8) per_cu = 2;
+    int per_cu = env ? atoi(env) : 1;
+    if (per_cu < 1 || per_cu > 8) per_cu = 1;
     int64_t want = (int64_t)per_cu * num_cus() / n_units;
     if (want < 1) want = 1;
-    if (want > MERGE_MAX_SPLITS) want = MERGE_MAX_SPLITS;
-    int64_t per = (n_keys + want - 1) / want;
-    per = ((per + step - 1) / step) * step;
+    if (want > MERGE_MAX_SPLITS / 2) want = MERGE_MAX_SPLITS / 2;
+    int64_t per = (n_keys / want) / step * step;
     if (per < step) per = step;
     const int n_splits = (int)((n_keys + per - 1) / per);
     const size_t acc_bytes = (size_t)n_splits * n_heads * HD * sizeof(float);
