@@ -679,14 +679,13 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
     // must be the short ones).  A block costs its number of key tiles, and 1.6 times that in the
     // PRECISE variant: rank r = item / n_kv_heads in the merge of the two descending sequences
     // 10 (p+1), p >= n_prec, and 16 (p+1), p < n_prec.
+    // The first item of a workgroup is its own index, without a ticket: read-modify-writes of one
+    // address from all XCDs are served one after the other (about 0.15 us each), so a first
+    // draw by every workgroup at once would start the last of them tens of microseconds late.
+    // Later draws come one by one as the items end.
     const uint32_t total = (uint32_t)(pblocks * n_kv_heads);
+    uint32_t item = blockIdx.x;
     for (;;) {
-        // nothing of the last item may still be on its way into LDS
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (threadIdx.x == 0) sh_item = atomicAdd(&tickets[0], 1u);
-        __syncthreads();
-        const uint32_t item = sh_item;
-        __syncthreads();                                 // everybody has the item, and is done with the last one's LDS
         if (item >= total) break;
         const int64_t rank = (int64_t)item / n_kv_heads;
         const int kvh = (int)(item % (uint32_t)n_kv_heads);
@@ -701,6 +700,12 @@ gqa_prefill_kernel(const uint16_t *__restrict__ K, const uint16_t *__restrict__ 
         if (pblk < 0) pblk = pblocks - 1 - (rank - before);
         if (pblk < n_prec) gqa_prefill_body<GROUP, true>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
         else gqa_prefill_body<GROUP, false>(smem_raw, K, V, Q, pos0, n, n_kv_heads, scale_log2e, out, pblk, kvh);
+        // nothing of the last item may still be on its way into LDS
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0) sh_item = gridDim.x + atomicAdd(&tickets[0], 1u);
+        __syncthreads();
+        item = sh_item;
+        __syncthreads();                                 // everybody has the item, and is done with the last one's LDS
     }
     // the last workgroup to leave puts the counters back to zero for the next launch (every
     // workgroup has drawn its last ticket before it counts itself out)
