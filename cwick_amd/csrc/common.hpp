@@ -68,6 +68,7 @@ int launch_indexer_scores(const uint8_t *keys, const float *kscale, int64_t key_
 struct IndexerBandRow {
     uint32_t n_cand;      // keys inside the band (may exceed the list's capacity)
     uint32_t fallback;    // the band could not be formed (bound not finite, NaN threshold)
+    uint32_t pad[30];     // a row to a 128-byte line: the workgroups of different rows add to n_cand at the same time
 };
 constexpr int CWICK_INDEXER_BAND_CAP = 4096;   // candidate list entries per row
 constexpr int CWICK_INDEXER_APPROX_KEYS = 2048;   // keys per workgroup (= per bound slot) of the approximate kernel

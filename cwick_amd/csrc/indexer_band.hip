@@ -307,7 +307,9 @@ indexer_rescore_kernel(const uint8_t *__restrict__ keys, const float *__restrict
     // front of the key's bytes): an entry past the end of the list is whatever the workspace
     // held, so it is clamped to a key of the row; what is computed for it is not stored.
     int64_t t_guess = cand[(size_t)b * cap + c0 + j];
-    const IndexerBandRow st = rows[b];
+    IndexerBandRow st;                                              // the two words in use, not the padding
+    st.n_cand = rows[b].n_cand;
+    st.fallback = rows[b].fallback;
     t_guess = t_guess < 0 ? 0 : (t_guess >= n_keys ? n_keys - 1 : t_guess);
     if (indexer_band_failed(st, cap)) {
         // the row did not fit the band: the workgroups of this launch score all of its keys

@@ -722,7 +722,9 @@ topk_band_finish_kernel(const float *__restrict__ scores, int64_t n, int64_t k, 
         v[j] = sc[i < n ? i : n - 1];
     }
     const uint32_t hi_part = tid < n_wg ? hi_count[(size_t)row * TOPK_MW_MAX_WGS + tid] : 0u;
-    const IndexerBandRow st = rows[row];
+    IndexerBandRow st;                                          // the two words in use, not the padding
+    st.n_cand = rows[row].n_cand;
+    st.fallback = rows[row].fallback;
     if (indexer_band_failed(st, cap)) {
         // the row did not fit the band: its scores are the exact kernel's by now, and its first
         // workgroup selects from all of them
