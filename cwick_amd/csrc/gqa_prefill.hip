@@ -99,28 +99,6 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     const int64_t q_stride = (int64_t)n_heads * PF_HD;
     const int64_t n_keys_all = pos0 + n;
 
-    // this lane's two query rows (column blocks A and B of the wave)
-    int64_t t_row[2], my_limit[2];
-    int j_row[2];
-    bool row_live[2];
-    bf16x8 qf[2][16];                       // B operand: lane (row, g) holds dims 16ks+8g .. +8
-                                            // (qf[1][PF_QX0..15] only pass through, see PfSmem::qx)
-#pragma unroll
-    for (int c = 0; c < 2; c++) {
-        const int r = wave * 64 + 32 * c + l32;
-        j_row[c] = r / P;
-        t_row[c] = t0 + (r % P);
-        row_live[c] = t_row[c] < n;
-        const int64_t tq = row_live[c] ? t_row[c] : n - 1;
-        my_limit[c] = pos0 + tq;
-        const uint16_t *qrow = Q + tq * q_stride + (size_t)(kvh * GROUP + j_row[c]) * PF_HD + 8 * g;
-#pragma unroll
-        for (int ks = 0; ks < 16; ks++)
-            qf[c][ks] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qrow + 16 * ks));
-    }
-#pragma unroll
-    for (int ks = PF_QX0; ks < 16; ks++) sm.qx[wave][ks - PF_QX0][lane] = __builtin_bit_cast(u32x4, qf[1][ks]);
-
     // keys 0 .. last position of the block (clipped to the chunk)
     int64_t last_t = t0 + P - 1;
     if (last_t > n - 1) last_t = n - 1;
@@ -153,6 +131,37 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
 #pragma unroll
         for (int i = 0; i < 4; i++) copy_one(src, lds_tile, i);
     };
+
+    // The first tiles are requested before the query rows: one trip to memory for all of them
+    // instead of one for Q, one for tile 0 and one for tile 1 (K has two buffers, V at least two).
+    issue(Kg, lds_k, 0);
+    issue(Vg, lds_v, 0);
+    if (n_tiles > 1) {
+        issue(Kg, lds_k + PF_TILE, 1);
+        if (!precise) issue(Vg, lds_v + PF_TILE, 1);
+    }
+
+    // this lane's two query rows (column blocks A and B of the wave)
+    int64_t t_row[2], my_limit[2];
+    int j_row[2];
+    bool row_live[2];
+    bf16x8 qf[2][16];                       // B operand: lane (row, g) holds dims 16ks+8g .. +8
+                                            // (qf[1][PF_QX0..15] only pass through, see PfSmem::qx)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int r = wave * 64 + 32 * c + l32;
+        j_row[c] = r / P;
+        t_row[c] = t0 + (r % P);
+        row_live[c] = t_row[c] < n;
+        const int64_t tq = row_live[c] ? t_row[c] : n - 1;
+        my_limit[c] = pos0 + tq;
+        const uint16_t *qrow = Q + tq * q_stride + (size_t)(kvh * GROUP + j_row[c]) * PF_HD + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            qf[c][ks] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qrow + 16 * ks));
+    }
+#pragma unroll
+    for (int ks = PF_QX0; ks < 16; ks++) sm.qx[wave][ks - PF_QX0][lane] = __builtin_bit_cast(u32x4, qf[1][ks]);
 
     // K fragment of k-step ks: block ks, slot 32g + (l32 ^ 8g)
     const uint32_t kfrag_off = (uint32_t)((32 * g + (l32 ^ (g << 3))) * 16);
@@ -353,12 +362,9 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
     };
 
     if constexpr (PRECISE) {
-        // ---- prologue: K(0), V(0), K(1); scores and softmax of tile 0 (sets the reference) ----
-        issue(Kg, lds_k, 0);
-        issue(Vg, lds_v, 0);
+        // ---- prologue: K(0), V(0), K(1) are on their way; scores and softmax of tile 0 (sets the reference) ----
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         PF_LDS_BARRIER();
-        if (n_tiles > 1) issue(Kg, lds_k + PF_TILE, 1);
 
         u32x4 pw[2][2], pl[2][2];
         {
@@ -520,16 +526,10 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
             if (t + 2 < n_tiles) issue(Vg, lds_v + (uint32_t)(((t + 2) % 3) * PF_TILE), t + 2);
         };
 
-        // prologue: K(0), V(0), K(1), V(1), K(2); scores and softmax of tile 0 (sets the reference),
+        // prologue (K(0), V(0), K(1), V(1) are on their way), K(2); scores and softmax of tile 0 (sets the reference),
         // scores of tile 1.  From then on step t fetches K(t+3) and V(t+2).
-        issue(Kg, lds_k, 0);
-        issue(Vg, lds_v, 0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // K(0), V(0), K(1), V(1)
         PF_LDS_BARRIER();
-        if (n_tiles > 1) {
-            issue(Kg, lds_k + PF_TILE, 1);
-            issue(Vg, lds_v + PF_TILE, 1);
-        }
         u32x4 pa[2][2], pb[2][2], pl[2][2];
         f32x16 sa[2], sb[2];
         scores(0, sa, -1, -1);
