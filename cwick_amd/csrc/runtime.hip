@@ -786,6 +786,36 @@ int cwick_hip_gqa_decode_sel(cwick_hip_kv *c, const int32_t *sel, int64_t n_list
     return st.out(out, dout, ob) && st.wait() ? 1 : 0;
 }
 
+int cwick_hip_mm_select(cwick_hip_kv *idx, int64_t limit, const float *iq, int index_heads, int block,
+                        int keep_blocks, int32_t *blk_out, int32_t *sel, int64_t max_sel, int64_t *n_sel) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    CWICK_REQUIRE(idx && iq && sel, "mm_select: null argument");
+    CWICK_REQUIRE(idx->n_kv_heads == 1, "mm_select: the index keys are a cache of one head per position, not %d",
+                  idx->n_kv_heads);
+    CWICK_REQUIRE(limit >= 1 && limit <= idx->capacity, "mm_select: limit %lld, capacity %lld", (long long)limit,
+                  (long long)idx->capacity);
+    CWICK_REQUIRE(index_heads >= 1 && index_heads <= 8, "mm_select: %d index heads (1..8)", index_heads);
+    CWICK_REQUIRE(keep_blocks >= 1 && keep_blocks <= 4096 && max_sel >= 1 && max_sel <= ((int64_t)1 << 24),
+                  "mm_select: blocks kept %d, max_sel %lld", keep_blocks, (long long)max_sel);
+    size_t qb = (size_t)index_heads * idx->head_dim * 4, scb = (size_t)limit * 4, bb = (size_t)(keep_blocks + 1) * 4;
+    size_t sb = (size_t)max_sel * 4;
+    Stager st(idx->ctx, pad256(qb) + pad256(scb) + pad256(bb) + pad256(sb) + 256);
+    CWICK_REQUIRE(st.ok, "mm_select: staging allocation failed");
+    const float *dq = st.in(iq, qb);
+    CWICK_REQUIRE(dq, "mm_select: upload failed");
+    float *dsc = st.room<float>(scb);
+    int32_t *dblk = st.room<int32_t>(bb), *dsel = st.room<int32_t>(sb), *dn = st.room<int32_t>(256);
+    if (!launch_mm_select(idx->k, dq, 1, limit, index_heads, idx->head_dim, block, keep_blocks, dsc, limit, dblk, dsel,
+                          max_sel, dn, idx->ctx.stream))
+        return 0;
+    int32_t got = 0;
+    if (blk_out && !st.out(blk_out, dblk, bb)) return 0;
+    if (!st.out(sel, dsel, sb) || !st.out(&got, dn, 4) || !st.wait()) return 0;
+    if (n_sel) *n_sel = got;
+    return 1;
+}
+
 int cwick_hip_gqa_prefill(cwick_hip_kv *c, int64_t pos0, int64_t n, const uint16_t *q, int n_heads,
                           float scale, float *out) {
     clear_error();

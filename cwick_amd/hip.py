@@ -94,6 +94,7 @@ SIGNATURES = {
     "cwick_hip_ikeys_pool_append_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _flt, _int, _vp, _vp]),
     "cwick_hip_candidate_select_dev": (_int, [_vp, _int, _i64, _int, _i64, _vp, _vp]),
     "cwick_hip_candidate_apply_dev": (_int, [_vp, _vp, _int, _i64, _vp]),
+    "cwick_hip_mm_select": (_int, [_vp, _i64, _vp, _int, _int, _int, _vp, _vp, _i64, _vp]),
     "cwick_hip_mm_select_dev": (_int, [_vp, _vp, _int, _i64, _int, _int, _int, _int, _vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "cwick_hip_latent_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
     "cwick_hip_ikeys_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
@@ -563,6 +564,17 @@ def gqa_prepare_dev(q_proj, q_head_stride, k_proj, v_proj, n, pos0, n_heads, n_k
 def candidate_select_dev(scores, batch, n, block, keep_blocks, cand, stream=None, raw=False):
     rc = lib().cwick_hip_candidate_select_dev(_dp(scores), batch, n, block, keep_blocks, _dp(cand), stream)
     return rc if raw else _check(rc, "candidate_select_dev")
+
+
+def mm_select(idx_cache, limit, iq, block, keep_blocks, max_sel):
+    """One query, host operands: -> (blocks, positions) as the reference leaves them."""
+    iq, iqp = _np(iq, np.float32)
+    blk = np.empty(keep_blocks + 1, np.int32)
+    sel = np.empty(max_sel, np.int32)
+    ns = _i64(0)
+    _check(lib().cwick_hip_mm_select(idx_cache.h, limit, iqp, iq.shape[0], block, keep_blocks, blk.ctypes.data,
+                                     sel.ctypes.data, max_sel, C.byref(ns)), "mm_select")
+    return blk[blk >= 0], sel[:ns.value]
 
 
 def mm_select_dev(idx_keys, iq, batch, limit0, index_heads, index_dim, block, keep_blocks, scores, score_stride,

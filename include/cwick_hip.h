@@ -402,6 +402,15 @@ int cwick_hip_gqa_decode_sel_dev(const uint16_t *k, const uint16_t *v, int64_t n
  * cwick_hip_gqa_decode_sel_dev takes with n_list = max_sel), n_sel int32
  * [batch] (out, may be NULL).  1..8 index heads, index_dim a multiple of 8 up
  * to 512, at most 16383 blocks. */
+/* The same for one query of an engine whose state is in host memory: the index
+ * keys are the K side of a cwick_hip_kv created with one head per position
+ * (cwick_hip_kv_create(capacity, 1, index_dim); rows appended with
+ * cwick_hip_kv_write, the V side unused), iq, blk_out (may be NULL), sel and
+ * n_sel (may be NULL) are host pointers.  sel then feeds
+ * cwick_hip_gqa_decode_sel with n_list = *n_sel. */
+int cwick_hip_mm_select(cwick_hip_kv *idx, int64_t limit, const float *iq, int index_heads,
+                        int block, int keep_blocks, int32_t *blk_out, int32_t *sel,
+                        int64_t max_sel, int64_t *n_sel);
 int cwick_hip_mm_select_dev(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0,
                             int index_heads, int index_dim, int block, int keep_blocks,
                             float *scores, int64_t score_stride, int32_t *blk_out,

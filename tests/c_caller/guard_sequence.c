@@ -191,6 +191,61 @@ int main(void) {
     cpu_gqa(kb, vb, GK, GKV, GD, gq, GH, 0.0625f, gref);
     ok &= cwick_hip_gqa_decode(kv, GK, gq, GH, 0.0625f, go) && check("gqa_decode (GPU)", go, gref, GH * GD);
     ok &= cwick_hip_gqa_decode(kv, GK + 1, gq, GH, 0.0625f, go) == 0;       /* past the capacity: declined */
+
+    /* ---- block-sparse decode: the selection of src/mm_model.c:1733-1780 and :1969-1976, then the
+     * attention over the kept positions (:1962-2047), against this file's own loops ---- */
+    {
+        enum { IH = 4, ID = 128, BS = 64, KEEP = 3, MAXSEL = (KEEP + 1) * BS };
+        uint16_t *ik = malloc(sizeof(uint16_t) * GK * ID);
+        float *iq = malloc(sizeof(float) * IH * ID), *isc = malloc(sizeof(float) * GK);
+        for (int i = 0; i < GK * ID; i++) ik[i] = f32_to_bf16(frand());
+        for (int i = 0; i < IH * ID; i++) iq[i] = frand();
+        cwick_hip_kv *idx = cwick_hip_kv_create(GK, 1, ID);
+        if (!idx) { printf("FAIL kv_create (index keys): %s\n", cwick_hip_last_error()); return 1; }
+        ok &= cwick_hip_kv_write(idx, 0, GK, ik, ik);
+        for (int s = 0; s < GK; s++) {                      /* mm_index_scores */
+            float tot = 0.0f;
+            for (int h = 0; h < IH; h++) {
+                float d = 0.0f;
+                for (int i = 0; i < ID; i++) d = fmaf(iq[h * ID + i], bf16_to_f32(ik[s * ID + i]), d);
+                if (d > 0.0f) tot += d;
+            }
+            isc[s] = tot;
+        }
+        enum { NBLK = (GK + BS - 1) / BS };
+        float bmax[NBLK];
+        int chosen[NBLK] = {0}, want_blk[KEEP + 1], nb = 0;
+        for (int b = 0; b < NBLK; b++) {
+            bmax[b] = -1e30f;
+            for (int s = b * BS; s < (b + 1) * BS && s < GK; s++) bmax[b] = fmaxf(bmax[b], isc[s]);
+        }
+        for (int r = 0; r < KEEP; r++) {                    /* the KEEP best blocks (scores are tie-free here) */
+            int best = -1;
+            for (int b = 0; b < NBLK; b++) if (!chosen[b] && (best < 0 || bmax[b] > bmax[best])) best = b;
+            chosen[best] = 1;
+        }
+        chosen[GK / BS] = 1;                                /* the newest block, always */
+        for (int b = 0; b < NBLK; b++) if (chosen[b]) want_blk[nb++] = b;
+        int32_t want_pos[MAXSEL], got_blk[KEEP + 1], got_pos[MAXSEL];
+        int64_t n_want = 0, n_got = -1;
+        for (int i = 0; i < nb; i++)
+            for (int s = want_blk[i] * BS; s < (want_blk[i] + 1) * BS && s < GK; s++) want_pos[n_want++] = s;
+        int sel_ok = cwick_hip_mm_select(idx, GK, iq, IH, BS, KEEP, got_blk, got_pos, MAXSEL, &n_got) && n_got == n_want;
+        for (int i = 0; sel_ok && i < nb; i++) sel_ok &= got_blk[i] == want_blk[i];
+        for (int64_t i = 0; sel_ok && i < n_want; i++) sel_ok &= got_pos[i] == want_pos[i];
+        printf("%-34s %s (%lld positions in %d blocks)\n", "mm_select (GPU)", sel_ok ? "equal" : "DIFFERS",
+               (long long)n_want, nb);
+        ok &= sel_ok;
+        uint16_t *kg = malloc(sizeof(uint16_t) * MAXSEL * GKV * GD), *vg = malloc(sizeof(uint16_t) * MAXSEL * GKV * GD);
+        for (int64_t i = 0; i < n_want; i++) {
+            memcpy(kg + i * GKV * GD, kb + (size_t)want_pos[i] * GKV * GD, sizeof(uint16_t) * GKV * GD);
+            memcpy(vg + i * GKV * GD, vb + (size_t)want_pos[i] * GKV * GD, sizeof(uint16_t) * GKV * GD);
+        }
+        cpu_gqa(kg, vg, (int)n_want, GKV, GD, gq, GH, 0.0625f, gref);
+        ok &= cwick_hip_gqa_decode_sel(kv, got_pos, n_got, gq, GH, 0.0625f, go) &&
+              check("gqa_decode_sel over them (GPU)", go, gref, GH * GD);
+        cwick_hip_kv_free(idx);
+    }
     cwick_hip_kv_free(kv);
     cwick_hip_shutdown();
     printf(ok ? "OK\n" : "FAILED\n");

@@ -1180,3 +1180,31 @@ def test_mm_block_sparse_decode_chain(hip, orc, n_rows, nh, nkv, hd):
     dense = hip.gqa_decode(cache, n_rows, c["q"], c["scale"])
     assert_close(dense, orc.gqa_decode(c["q"], c["k"], c["v"], c["scale"], nthreads=0), "gqa decode group 16")
     cache.free()
+
+
+def test_mm_select_host_operands(hip, orc):
+    """The block selection for an engine whose state is in host memory: index keys kept as the K
+    side of a one-head cache handle, everything else host pointers, then the attention over the
+    returned positions (src/mm_model.c:1962-2047)."""
+    say("[case] mm select, host operands")
+    n, ih, idim, bs, keep, nh, nkv, hd = 3000, 4, 128, 128, 16, 64, 4, 128
+    g = synth.rng(5150)
+    keys = synth.normal_bf16(g, (n, idim))
+    iq = g.standard_normal((ih, idim)).astype(np.float32)
+    idx = hip.KVCache(n, 1, idim)
+    idx.write(0, keys, keys)
+    for limit in (n, 2944, 1):                      # a partly filled newest block, a full one, a single position
+        blk, pos = hip.mm_select(idx, limit, iq, bs, keep, 4096)
+        rblk, rpos = orc.mm_select_blocks(orc.mm_index_scores(iq, keys, limit), limit, bs, keep, 4096)
+        assert list(blk) == list(rblk) and list(pos) == list(rpos), limit
+    blk, pos = hip.mm_select(idx, n, iq, bs, keep, 4096)
+    c = synth.cfg1_gqa_decode(n, nh, nkv, hd, seed=5151)
+    kv = hip.KVCache(n, nkv, hd)
+    kv.write(0, c["k"].reshape(n, -1), c["v"].reshape(n, -1))
+    got = hip.gqa_decode_sel(kv, pos.astype(np.int32), c["q"], c["scale"])
+    ref = orc.gqa_decode(c["q"], c["k"][pos], c["v"][pos], c["scale"])
+    assert_close(got, ref, "block-sparse decode, host operands, %d positions" % pos.size)
+    with pytest.raises(hip.Declined):
+        hip.mm_select(kv, n, iq, bs, keep, 4096)    # four heads per position: not an index-key cache
+    idx.free()
+    kv.free()
