@@ -95,3 +95,25 @@ def test_dsa_decode_under_graph_capture(hip):
     def call(sp):
         hip.dsa_decode_dev(ik, iks, 0, 0, rows, scales, 0, 0, B, N, qi, w, 64, K, q, 128, c["scale"], tmp, sel, out, sp)
     _replay_equals_eager(torch, call, qi, out, s, "dsa_decode_dev")
+
+
+def test_block_sparse_decode_under_graph_capture(hip):
+    import torch
+    print("[case] graph capture: mm_select_dev -> gqa_decode_sel_dev", flush=True)
+    n, nh, nkv, hd, ih, idim, bs, keep = 5000, 64, 4, 128, 4, 128, 128, 16
+    g = synth.rng(3104)
+    c = synth.cfg1_gqa_decode(n, nh, nkv, hd, seed=3105)
+    d = lambda a: torch.from_numpy(a.view(np.int16)).cuda()
+    k, v, q = d(c["k"]), d(c["v"]), d(c["q"])
+    keys = d(synth.normal_bf16(g, (n, idim)))
+    iq = torch.from_numpy(g.standard_normal((ih * idim // 8, 8)).astype(np.float32)).cuda()   # pieces of eight dims are permuted
+    max_sel = (keep + 1) * bs
+    sc = torch.empty((1, n), dtype=torch.float32, device="cuda")
+    sel = torch.empty((1, max_sel), dtype=torch.int32, device="cuda")
+    out = torch.empty((nh, hd), dtype=torch.float32, device="cuda")
+    s = torch.cuda.Stream()
+
+    def call(sp):
+        hip.mm_select_dev(keys, iq, 1, n, ih, idim, bs, keep, sc, n, None, sel, max_sel, None, sp)
+        hip.gqa_decode_sel_dev(k, v, n, nkv, hd, sel, max_sel, q, nh, c["scale"], out, sp)
+    _replay_equals_eager(torch, call, iq, out, s, "mm_select_dev -> gqa_decode_sel_dev")
