@@ -5,12 +5,13 @@
 // positions (:1969-1976).  What leaves is a position list per query, padded with -1, that
 // launch_gqa_decode takes as its `sel`: the whole selection stays on the device.
 //
-//   1. mm_index_scores_kernel   one thread per position: for every index head the dot of the
-//      head's fp32 query with the position's bf16 key, a fused multiply-add per dimension in
-//      dimension order from zero (the reference's serial loop), ReLU, the heads added in head
-//      order.  The query is read through the scalar unit; a thread requests its whole
-//      256-byte key row in 16-byte pieces before it uses the first (the serial order ties a key
-//      to one thread, so the row cannot be spread over lanes).
+//   1. mm_index_scores_kernel   one thread per (position, index head): the dot of the head's fp32
+//      query with the position's bf16 key, a fused multiply-add per dimension in dimension order
+//      from zero (the reference's serial loop: a chain belongs to one thread, but the heads of a
+//      position are independent chains), then ReLU and the heads added in head order by the
+//      first wave.  A workgroup is 64 positions x one wave per head; a wave's query is uniform
+//      and read through the scalar unit; a thread requests its whole 256-byte key row in
+//      16-byte pieces before it uses the first.
 //   2. mm_blockmax_kernel       one wave per block: the largest score inside the block, started
 //      from -1e30 like the reference; blocks past a query's last one get -inf so that rows of
 //      a chunk with different block counts share one top-k launch.
@@ -27,12 +28,70 @@ namespace cwick {
 namespace {
 
 constexpr int MM_THREADS = 256;
-constexpr int MM_SCORE_THREADS = 64;        // one wave: a short context still spreads over many CUs
+constexpr int MM_SCORE_THREADS = 64;        // positions per workgroup of the scoring kernel (one wave per index head)
 constexpr int MM_MAX_HEADS = 8;
+constexpr int64_t MM_SHORT_POSITIONS = 32768;   // up to here the scoring kernel takes a wave per head
 constexpr int MM_MAX_DIM = 512;
 
-__global__ void __launch_bounds__(MM_SCORE_THREADS)
+__global__ void __launch_bounds__(MM_SCORE_THREADS * MM_MAX_HEADS)
 mm_index_scores_kernel(const uint16_t *__restrict__ keys, const float *__restrict__ iq, int64_t limit0, int ih, int id,
+                       float *__restrict__ scores, int64_t score_stride) {
+    // workgroup = 64 positions x ih waves: wave h runs head h's chain for the 64 positions (the
+    // heads are independent until the sum), its lanes the positions
+    __shared__ float sh_d[MM_MAX_HEADS][MM_SCORE_THREADS];
+    const int row = blockIdx.y;
+    const int64_t limit = limit0 + row;
+    if ((int64_t)blockIdx.x * MM_SCORE_THREADS >= limit) return;          // the whole workgroup: before the barrier
+    const int lane = threadIdx.x & 63;
+    const int h = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t s = (int64_t)blockIdx.x * MM_SCORE_THREADS + lane;
+    const int64_t sc = s < limit ? s : limit - 1;                   // threads past the end read the last row
+    const u32x4 *kp = (const u32x4 *)(keys + (size_t)sc * id);
+    const int chunks = id / 8;
+    // sixteen pieces of the row (a whole 128-dimension key) are requested before the first is
+    // used: one round trip to memory per key
+    constexpr int G = 16;
+    u32x4 kw[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) kw[g] = kp[g < chunks ? g : chunks - 1];
+    // the head's query is the same for every lane of the wave: its address is uniform, so it
+    // arrives through the scalar unit, eight values a load, and enters the multiply-adds as a
+    // scalar operand
+    const float *__restrict__ q = iq + ((size_t)row * ih + h) * id;
+    float d = 0.0f;
+    for (int c0 = 0; c0 < chunks; c0 += G) {
+        if (c0) {
+#pragma unroll
+            for (int g = 0; g < G; g++) kw[g] = kp[c0 + g < chunks ? c0 + g : chunks - 1];
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            if (c0 + g < chunks) {                                  // uniform
+                const float *qc = q + (c0 + g) * 8;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    d = __builtin_fmaf(qc[2 * i], bf16lo_to_f32(kw[g][i]), d);
+                    d = __builtin_fmaf(qc[2 * i + 1], bf16hi_to_f32(kw[g][i]), d);
+                }
+            }
+        }
+    }
+    sh_d[h][lane] = d;
+    __syncthreads();
+    if (h != 0) return;
+    float tot = 0.0f;
+    for (int j = 0; j < ih; j++) {
+        const float dj = sh_d[j][lane];
+        if (dj > 0.0f) tot = tot + dj;
+    }
+    if (s < limit) scores[(size_t)row * score_stride + s] = tot;
+}
+
+// The same for long contexts: one thread per position runs the chains of all heads (a key row is
+// read by one wave instead of one per head, which is what counts once the rows come from HBM
+// rather than out of a cache that the head waves share).
+__global__ void __launch_bounds__(MM_SCORE_THREADS)
+mm_index_scores_long_kernel(const uint16_t *__restrict__ keys, const float *__restrict__ iq, int64_t limit0, int ih, int id,
                        float *__restrict__ scores, int64_t score_stride) {
     const int row = blockIdx.y;
     const int64_t limit = limit0 + row;
@@ -179,9 +238,16 @@ int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64
     int32_t *blk = (int32_t *)(ws + bsc_b);
     {
         ProfScope ps(CWICK_HIP_PROF_MM_SELECT, s);
-        mm_index_scores_kernel<<<dim3((unsigned)((limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS), batch),
-                                 MM_SCORE_THREADS, 0, s>>>(idx_keys, iq, limit0, index_heads, index_dim, scores,
-                                                            score_stride);
+        const dim3 sgrid((unsigned)((limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS), batch);
+        // up to 32 K positions a wave per head (8 192 positions: 8.5 -> 5.5 us); beyond, the head
+        // waves' reads of the same key rows cost more than their parallelism gains (262 144
+        // positions: 19 us against 32)
+        if (limit_max * batch <= MM_SHORT_POSITIONS)
+            mm_index_scores_kernel<<<sgrid, MM_SCORE_THREADS * index_heads, 0, s>>>(idx_keys, iq, limit0, index_heads,
+                                                                                index_dim, scores, score_stride);
+        else
+            mm_index_scores_long_kernel<<<sgrid, MM_SCORE_THREADS, 0, s>>>(idx_keys, iq, limit0, index_heads, index_dim,
+                                                                       scores, score_stride);
         mm_blockmax_kernel<<<dim3((unsigned)((nblk_max + 3) / 4), batch), MM_THREADS, 0, s>>>(scores, score_stride,
                                                                                           limit0, block, nblk_max, bsc);
     }
