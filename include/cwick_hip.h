@@ -480,7 +480,7 @@ enum {
     CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel, or in a fused select indexer_approx_kernel + topk_mw_hist_kernel + topk_mw_classify_kernel + indexer_rescore_kernel + the exact kernel's fallback pass */
     CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel; in a fused select topk_band_finish_kernel */
     CWICK_HIP_PROF_MLA_PREFILL,         /* mla_prefill64_kernel (chunked prefill of more than 64 heads) */
-    CWICK_HIP_PROF_MM_SELECT,           /* mm_index_scores_kernel + mm_blockmax_kernel + mm_expand_kernel (the block top-k between them counts under CWICK_HIP_PROF_TOPK) */
+    CWICK_HIP_PROF_MM_SELECT,           /* mm_index_scores[_long]_kernel + mm_pick_kernel; for block sizes that are not a multiple of 64 mm_blockmax_kernel and mm_expand_kernel, with the block top-k between them under CWICK_HIP_PROF_TOPK */
     CWICK_HIP_PROF_COUNT
 };
 void cwick_hip_prof_enable(int on);
