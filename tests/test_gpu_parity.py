@@ -1105,6 +1105,8 @@ def test_gqa_decode_over_selected_blocks(hip, orc, n_rows, nh, nkv, hd, bs, keep
     (1, 2, 4, 128, 128, 16, 4096),         # the first positions of a sequence
     (40000, 2, 8, 64, 64, 20, 1000),       # the list cut at max_sel
     (300, 1, 2, 512, 128, 16, 4096),       # more blocks asked for than exist
+    (70000, 1, 4, 128, 64, 16, 4096),      # more than 1024 blocks: the streaming row select inside the one-workgroup step
+    (9000, 3, 4, 128, 192, 5, 4096),       # blocks of three scoring groups
 ])
 def test_mm_select_blocks_on_device(hip, orc, limit0, batch, ih, idim, bs, keep, max_sel):
     """The block selection of the block-sparse decode (src/mm_model.c:1764-1780, :1733-1761,
