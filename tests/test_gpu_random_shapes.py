@@ -126,3 +126,43 @@ def test_prefill_random_chunks(hip, orc, seed):
         ref = orc.mla_prefill_chunk(c["q"], c["rows"], c["scales"], pos0, c["scale"], nthreads=0)
         assert_close(got, ref, "mla prefill pos0 %d n %d heads %d" % (pos0, n, nh))
         cache.free()
+
+
+@pytest.mark.parametrize("seed", [501])
+def test_mm_select_random_shapes(hip, orc, seed):
+    """The block selection of the block-sparse decode on random limits, chunk lengths, block
+    sizes (whole scoring groups and not), head counts and list caps: scores bit for bit, blocks
+    and positions equal to the oracle's."""
+    import torch
+    g = np.random.default_rng(seed)
+    s = torch.cuda.current_stream().cuda_stream
+    for _ in range(24):
+        bs = int(g.choice([64, 128, 192, 256, 7, 100, 33]))
+        limit0 = int(g.choice([g.integers(1, 300), g.integers(300, 9000), g.integers(9000, 80000)]))
+        batch = int(g.choice([1, 1, 2, 5]))
+        ih = int(g.integers(1, 9))
+        idim = int(g.choice([8, 64, 128, 256]))
+        keep = int(g.choice([1, 3, 16, 40]))
+        max_sel = int(g.choice([4096, 500, (keep + 1) * bs]))
+        say("[case] mm select random", limit0, batch, ih, idim, bs, keep, max_sel)
+        n = limit0 + batch - 1
+        keys = synth.normal_bf16(g, (n, idim))
+        iq = g.standard_normal((batch, ih, idim)).astype(np.float32)
+        d_keys = torch.from_numpy(keys.view(np.int16)).cuda()
+        d_iq = torch.from_numpy(iq).cuda()
+        d_sc = torch.empty((batch, n), dtype=torch.float32, device="cuda")
+        d_blk = torch.empty((batch, keep + 1), dtype=torch.int32, device="cuda")
+        d_sel = torch.empty((batch, max_sel), dtype=torch.int32, device="cuda")
+        d_ns = torch.empty((batch,), dtype=torch.int32, device="cuda")
+        hip.mm_select_dev(d_keys, d_iq, batch, limit0, ih, idim, bs, keep, d_sc, n, d_blk, d_sel, max_sel, d_ns, s)
+        torch.cuda.synchronize()
+        sc, blk, sel, ns = d_sc.cpu().numpy(), d_blk.cpu().numpy(), d_sel.cpu().numpy(), d_ns.cpu().numpy()
+        for t in range(batch):
+            limit = limit0 + t
+            ref_sc = orc.mm_index_scores(iq[t], keys, limit)
+            assert np.array_equal(sc[t, :limit].view(np.uint32), ref_sc.view(np.uint32)), "query %d: scores" % t
+            rblk, rpos = orc.mm_select_blocks(ref_sc, limit, bs, keep, max_sel)
+            assert list(blk[t, :rblk.size]) == list(rblk) and (blk[t, rblk.size:] == -1).all(), "query %d: blocks" % t
+            assert ns[t] == rpos.size and list(sel[t, :rpos.size]) == list(rpos) and (sel[t, rpos.size:] == -1).all(), \
+                "query %d: positions" % t
+
