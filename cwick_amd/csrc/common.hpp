@@ -30,11 +30,15 @@ bool hip_ok(hipError_t e, const char *what);   // records the error text on fail
 // ---- runtime ---------------------------------------------------------------
 bool backend_ready();                       // device 0 is up and selected
 int num_cus();
-// Grow-only scratch keyed by stream.  Valid until the next call on that stream
-// asks for more bytes; kernels enqueued earlier on the stream have finished
-// with it by the time a later enqueue on the same stream touches it.
-void *workspace(hipStream_t s, size_t bytes);
-uint32_t *ticket_counters(hipStream_t s);   // 64 dwords per stream, zero between kernels
+// Grow-only scratch keyed by stream and slot.  A call's buffer stays valid for the kernels it
+// enqueues (and for graphs captured from them) until the stream is released: growing allocates
+// a new buffer and retires the old one, it neither frees nor waits.  Returns null (reason
+// recorded) when it would have to allocate while the stream is being captured.
+// Slot WS_NESTED belongs to launchers that other launchers call with operands in slot WS_MAIN
+// (the top-k select inside the block selections).
+constexpr int WS_MAIN = 0, WS_NESTED = 1, WS_SLOTS = 2;
+void *workspace(hipStream_t s, size_t bytes, int slot = WS_MAIN);
+uint32_t *ticket_counters(hipStream_t s);   // 64 dwords per stream, zero between kernels; null under capture if not there yet
 
 // Phase timer: brackets the launches made while it is alive with two events on
 // `s` when profiling is enabled; does nothing (and records nothing) otherwise.

@@ -257,7 +257,7 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     const size_t acc_bytes = (size_t)n_splits * n_heads * HD * sizeof(float);
     const size_t ml_bytes = (size_t)n_splits * n_heads * 2 * sizeof(float);
     char *ws = (char *)workspace(s, acc_bytes + ml_bytes);
-    CWICK_REQUIRE(ws, "gqa_decode: workspace allocation failed");
+    if (!ws) return 0;                      // workspace() has recorded why
     float *part_acc = (float *)ws, *part_ml = (float *)(ws + acc_bytes);
     {
         ProfScope ps(CWICK_HIP_PROF_GQA_DECODE, s);

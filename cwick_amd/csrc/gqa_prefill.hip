@@ -754,7 +754,7 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
         n_prec++;
     }
     uint32_t *tickets = ticket_counters(s);
-    CWICK_REQUIRE(tickets, "gqa_prefill: ticket counters");
+    if (!tickets) return 0;                 // ticket_counters() has recorded why
     const int64_t items = pblocks * n_kv_heads;
     const int64_t wgs = items < num_cus() ? items : num_cus();      // the LDS of a compute unit holds one workgroup
     {

@@ -435,7 +435,7 @@ int launch_indexer_banded(const uint8_t *keys, const float *kscale, int64_t key_
     size_t off_cs = off_cand + (size_t)batch * cap * sizeof(int32_t);
     const size_t total = off_cs + (size_t)batch * cap * sizeof(float);
     char *ws = (char *)workspace(s, total);
-    CWICK_REQUIRE(ws, "indexer_banded: workspace allocation failed");
+    if (!ws) return 0;                      // workspace() has recorded why
     float *beta_slots = (float *)(ws + off_beta);
     IndexerBandRow *rows = (IndexerBandRow *)(ws + off_rows);
     uint32_t *hi_count = (uint32_t *)(ws + off_hi);

@@ -956,7 +956,7 @@ int run(Params &p, hipStream_t s, bool fixed = false) {
             if (!ws) return 0;
         } else {
             ws = (char *)workspace(s, acc_b + ml_b);
-            CWICK_REQUIRE(ws, "mla: workspace allocation failed");
+            if (!ws) return 0;                      // workspace() has recorded why
         }
         p.part_acc = (uint32_t *)ws;
         p.part_ml = (float *)(ws + acc_b);

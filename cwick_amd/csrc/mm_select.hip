@@ -287,15 +287,14 @@ int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64
     CWICK_REQUIRE(max_sel >= 1 && max_sel <= ((int64_t)1 << 24), "mm_select: max_sel %lld", (long long)max_sel);
     CWICK_REQUIRE(((uintptr_t)idx_keys) % 16 == 0, "mm_select: index keys must be 16-byte aligned");
     const int64_t nblk_max = (limit_max + block - 1) / block;
-    // rows this short are selected by the one-workgroup top-k kernels, which take no workspace:
-    // the block scores can sit in this call's
+    // (the top-k below keeps its own workspace slot, so the block scores can sit in this call's)
     CWICK_REQUIRE(nblk_max < 16384, "mm_select: %lld blocks (at most 16383)", (long long)nblk_max);
     const bool fused = block % MM_SCORE_THREADS == 0;          // a block is whole groups of the scoring kernel
     const int64_t ng_max = (limit_max + MM_SCORE_THREADS - 1) / MM_SCORE_THREADS;
     const size_t bsc_b = ((size_t)batch * nblk_max * 4 + 255) & ~(size_t)255;
     const size_t blk_b = ((size_t)batch * keep_blocks * 4 + 255) & ~(size_t)255;
     char *ws = (char *)workspace(s, bsc_b + blk_b + (fused ? (size_t)batch * ng_max * 4 : 0));
-    CWICK_REQUIRE(ws, "mm_select: workspace allocation failed");
+    if (!ws) return 0;                      // workspace() has recorded why
     float *bsc = (float *)ws;
     int32_t *blk = (int32_t *)(ws + bsc_b);
     float *gmax = fused ? (float *)(ws + bsc_b + blk_b) : nullptr;

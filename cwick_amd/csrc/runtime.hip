@@ -96,35 +96,61 @@ bool backend_ready() {
 int num_cus() { return g_cus > 0 ? g_cus : 256; }
 
 // ---------------------------------------------------------------------------
-// grow-only scratch, one pair of buffers per stream
+// grow-only scratch, WS_SLOTS buffers per stream
 // ---------------------------------------------------------------------------
+// A buffer that has been handed out is never freed while its stream is known to the library:
+// kernels already enqueued and HIP graphs captured earlier carry its address.  When a call
+// needs more, a new buffer is allocated and the old one is retired until
+// cwick_hip_stream_release() or cwick_hip_shutdown(); nothing waits for the stream.  Capacities at
+// least double, so the retired buffers of a stream add up to less than its current one.
 struct Scratch {
     void *p = nullptr;
     size_t cap = 0;
+    std::vector<void *> retired;
+    void free_all() {
+        if (p) (void)hipFree(p);
+        for (void *r : retired) (void)hipFree(r);
+        p = nullptr;
+        cap = 0;
+        retired.clear();
+    }
 };
-static std::unordered_map<hipStream_t, Scratch> g_ws;
+struct StreamScratch {
+    Scratch slot[WS_SLOTS];
+};
+static std::unordered_map<hipStream_t, StreamScratch> g_ws;
+
+// true (and the reason recorded) when `s` is being captured into a graph: nothing may be
+// allocated then, and the address of a buffer allocated now would end up in the graph
+static bool capturing(hipStream_t s, const char *what) {
+    if (!s) return false;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (st == hipStreamCaptureStatusNone) return false;
+    set_error("%s would have to allocate while the stream is being captured; run the shape once before the "
+              "capture or size the workspace with cwick_hip_reserve_dev", what);
+    return true;
+}
 
 static void *grow_one(Scratch &b, hipStream_t s, size_t bytes) {
     if (bytes <= b.cap) return b.p;
-    // A buffer in use by kernels already enqueued on `s` must outlive them.
-    if (b.p) {
-        if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize(workspace grow)")) return nullptr;
-        (void)hipFree(b.p);
-        b.p = nullptr;
-        b.cap = 0;
-    }
-    size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
-    if (!hip_ok(hipMalloc(&b.p, want), "hipMalloc(workspace)")) {
-        b.p = nullptr;
-        return nullptr;
-    }
+    if (capturing(s, "the split-K workspace")) return nullptr;
+    size_t want = bytes > 2 * b.cap ? bytes : 2 * b.cap;
+    want = (want + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    void *np = nullptr;
+    if (!hip_ok(hipMalloc(&np, want), "hipMalloc(workspace)")) return nullptr;
+    if (b.p) b.retired.push_back(b.p);
+    b.p = np;
     b.cap = want;
     return b.p;
 }
 
-void *workspace(hipStream_t s, size_t bytes) {
+void *workspace(hipStream_t s, size_t bytes, int slot) {
     std::lock_guard<std::mutex> lk(g_mu);
-    return grow_one(g_ws[s], s, bytes);
+    return grow_one(g_ws[s].slot[slot], s, bytes);
 }
 
 // A few dwords per stream that are zero whenever no kernel of the stream is running: kernels
@@ -134,9 +160,12 @@ uint32_t *ticket_counters(hipStream_t s) {
     std::lock_guard<std::mutex> lk(g_mu);
     auto it = g_tickets.find(s);
     if (it != g_tickets.end()) return it->second;
+    if (capturing(s, "the ticket counters")) return nullptr;
     void *p = nullptr;
     if (!hip_ok(hipMalloc(&p, 256), "hipMalloc(tickets)")) return nullptr;
-    if (!hip_ok(hipMemset(p, 0, 256), "hipMemset(tickets)")) {
+    // cleared on the stream whose kernels will count in them, and the clearing waited for
+    if (!hip_ok(hipMemsetAsync(p, 0, 256, s), "hipMemsetAsync(tickets)") ||
+        !hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize(tickets)")) {
         (void)hipFree(p);
         return nullptr;
     }
@@ -144,7 +173,7 @@ uint32_t *ticket_counters(hipStream_t s) {
     return (uint32_t *)p;
 }
 
-// forget (and free) the workspace of a stream that is about to be destroyed
+// forget (and free) what the library keeps for a stream that is about to be destroyed
 static void drop_workspace(hipStream_t s) {
     std::lock_guard<std::mutex> lk(g_mu);
     auto tk = g_tickets.find(s);
@@ -154,7 +183,7 @@ static void drop_workspace(hipStream_t s) {
     }
     auto it = g_ws.find(s);
     if (it == g_ws.end()) return;
-    if (it->second.p) (void)hipFree(it->second.p);
+    for (Scratch &b : it->second.slot) b.free_all();
     g_ws.erase(it);
 }
 
@@ -176,8 +205,7 @@ struct HostCtx {
             (void)hipStreamDestroy(stream);
             stream = nullptr;
         }
-        if (stage.p) (void)hipFree(stage.p);
-        stage = Scratch{};
+        stage.free_all();
     }
 };
 static std::mutex g_free_mu;
@@ -240,7 +268,8 @@ static void prof_drain_locked() {
 
 static void free_all_scratch() {
     std::lock_guard<std::mutex> lk(g_mu);
-    for (auto &kv : g_ws) if (kv.second.p) (void)hipFree(kv.second.p);
+    for (auto &kv : g_ws)
+        for (Scratch &b : kv.second.slot) b.free_all();
     g_ws.clear();
     for (auto &kv : g_tickets) (void)hipFree(kv.second);
     g_tickets.clear();
@@ -338,6 +367,38 @@ void cwick_hip_shutdown(void) {
         g_free_ctx.destroy();
     }
     free_all_scratch();
+}
+
+int cwick_hip_reserve_dev(void *stream, int64_t bytes) {
+    clear_error();
+    if (!backend_ready()) return 0;
+    CWICK_REQUIRE(bytes >= 0 && bytes <= ((int64_t)1 << 40), "reserve: %lld bytes", (long long)bytes);
+    hipStream_t s = (hipStream_t)stream;
+    // the main slot as asked; the nested one for the largest row the many-workgroup select takes
+    // (batch 64); the ticket counters of the prefill
+    if (bytes > 0 && !workspace(s, (size_t)bytes, WS_MAIN)) return 0;          // the reason is recorded
+    if (!workspace(s, topk_mw_workspace_bytes(64, 131072), WS_NESTED)) return 0;
+    if (!ticket_counters(s)) return 0;
+    return 1;
+}
+
+int64_t cwick_hip_workspace_bytes_dev(void *stream) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_ws.find((hipStream_t)stream);
+    return it == g_ws.end() ? 0 : (int64_t)it->second.slot[WS_MAIN].cap;
+}
+
+int cwick_hip_stream_release(void *stream) {
+    clear_error();
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (g_state != 1) return 1;                  // nothing was ever kept
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (capturing(s, "cwick_hip_stream_release")) return 0;
+    CWICK_HIP_CALL(hipStreamSynchronize(s));
+    drop_workspace(s);
+    return 1;
 }
 
 const char *cwick_hip_last_error(void) { return g_err; }

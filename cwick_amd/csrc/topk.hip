@@ -622,8 +622,9 @@ int launch_topk(const float *scores, int batch, int64_t n, int64_t k, int32_t *o
     const int64_t n_wg = topk_mw_wgs(n);
     if (n_wg >= 8 && n_wg <= TOPK_MW_MAX_WGS) {
         const size_t ws_row = topk_mw_row_dwords(n_wg, n_wg);       // dwords: slices, four states, above counts
-        uint32_t *ws = (uint32_t *)workspace(s, (size_t)batch * ws_row * sizeof(uint32_t));
-        CWICK_REQUIRE(ws, "topk: workspace allocation failed");
+        // its own slot: the callers that select among block scores keep those in the main one
+        uint32_t *ws = (uint32_t *)workspace(s, (size_t)batch * ws_row * sizeof(uint32_t), WS_NESTED);
+        if (!ws) return 0;                      // workspace() has recorded why
         const dim3 grid((unsigned)n_wg, (unsigned)batch);
         ProfScope ps(CWICK_HIP_PROF_TOPK, s);
         for (int pass = 0; pass < 4; pass++)

@@ -98,6 +98,9 @@ SIGNATURES = {
     "cwick_hip_mm_select_dev": (_int, [_vp, _vp, _int, _i64, _int, _int, _int, _int, _vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "cwick_hip_latent_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
     "cwick_hip_ikeys_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
+    "cwick_hip_reserve_dev": (_int, [_vp, _i64]),
+    "cwick_hip_workspace_bytes_dev": (_i64, [_vp]),
+    "cwick_hip_stream_release": (_int, [_vp]),
     "cwick_hip_probe_hbm_read": (_int, [C.c_size_t, _int, C.POINTER(C.c_double)]),
     "cwick_hip_probe_mfma": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "cwick_hip_e4m3_table": (_int, [_vp]),
@@ -496,11 +499,10 @@ def gqa_prefill_dev(k, v, pos0, n, n_kv_heads, head_dim, q, n_heads, scale, out,
 
 
 def mla_decode_dev(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list, q,
-                   n_heads, scale, out, stream=None):
-    return _check(lib().cwick_hip_mla_decode_dev(_dp(rows), _dp(scales), row_bstride,
-                                                 scale_bstride, n_rows, batch, _dp(sel), n_list,
-                                                 _dp(q), n_heads, scale, _dp(out), stream),
-                  "mla_decode_dev")
+                   n_heads, scale, out, stream=None, raw=False):
+    rc = lib().cwick_hip_mla_decode_dev(_dp(rows), _dp(scales), row_bstride, scale_bstride, n_rows, batch,
+                                        _dp(sel), n_list, _dp(q), n_heads, scale, _dp(out), stream)
+    return rc if raw else _check(rc, "mla_decode_dev")
 
 
 def mla_decode_static_dev(rows, scales, row_bstride, scale_bstride, n_rows, batch, sel, n_list, q,
@@ -583,6 +585,20 @@ def mm_select_dev(idx_keys, iq, batch, limit0, index_heads, index_dim, block, ke
                                        keep_blocks, _dp(scores), score_stride, _dp(blk_out), _dp(sel), max_sel,
                                        _dp(n_sel), stream)
     return rc if raw else _check(rc, "mm_select_dev")
+
+
+def reserve_dev(stream, nbytes, raw=False):
+    rc = lib().cwick_hip_reserve_dev(stream, nbytes)
+    return rc if raw else _check(rc, "reserve_dev")
+
+
+def workspace_bytes_dev(stream):
+    return int(lib().cwick_hip_workspace_bytes_dev(stream))
+
+
+def stream_release(stream, raw=False):
+    rc = lib().cwick_hip_stream_release(stream)
+    return rc if raw else _check(rc, "stream_release")
 
 
 def candidate_apply_dev(scores, cand, batch, n, stream=None):

@@ -246,8 +246,33 @@ int cwick_hip_dsa_decode(cwick_hip_ikeys *ik, cwick_hip_latent *lat, int slot0, 
 /* ---- the same operations on HBM-resident operands ---------------------- */
 /* All pointers are device pointers; `stream` is a hipStream_t (NULL = the
  * null stream).  Kernels are enqueued, nothing is copied or waited for.
- * Scratch for split-K partials comes from a grow-only per-device workspace
- * inside the library. */
+ * Scratch (split-K partials, select state) comes from a grow-only workspace
+ * that the library keeps per stream.  A call whose shape needs more than the
+ * stream's workspace holds allocates a larger buffer (hipMalloc) and keeps the
+ * old one until cwick_hip_stream_release() or cwick_hip_shutdown(): kernels
+ * already enqueued and HIP graphs captured earlier stay valid, and no *_dev
+ * call ever waits for the stream or frees memory.  While the stream is being
+ * captured into a graph a call that would have to allocate declines instead
+ * (the capture stays intact): run each shape once before capturing, or size
+ * the workspace up front with cwick_hip_reserve_dev().  The split-K partials and the
+ * ticket counters of cwick_hip_gqa_prefill_dev belong to the stream: two calls
+ * that use one stream's workspace at the same time (a graph replayed on another stream
+ * while eager calls run on the capture stream) race. */
+
+/* No counterpart in the reference (its GPU hooks allocate on demand,
+ * src/metal.c:306-319): sizes the workspace of `stream` to at least `bytes`,
+ * together with the small fixed-size state the select and prefill kernels keep
+ * per stream, so that later *_dev calls whose scratch fits allocate nothing.
+ * cwick_hip_workspace_bytes_dev() reports what the stream holds now: run the
+ * largest shapes once and reserve that figure in the next process. */
+int cwick_hip_reserve_dev(void *stream, int64_t bytes);
+int64_t cwick_hip_workspace_bytes_dev(void *stream);
+/* Waits for `stream`, then frees everything the library keeps for it
+ * (workspace, retired buffers, ticket counters).  For callers about to destroy
+ * a stream they passed to *_dev calls: a later stream may reuse the handle
+ * value.  Graphs captured from this stream's calls must not be replayed
+ * afterwards. */
+int cwick_hip_stream_release(void *stream);
 
 int cwick_hip_gqa_decode_dev(const uint16_t *k, const uint16_t *v, int64_t n_keys,
                              int n_kv_heads, int head_dim, const uint16_t *q, int n_heads,
@@ -475,11 +500,11 @@ enum {
     CWICK_HIP_PROF_GQA_DECODE = 0,      /* gqa_decode_split_kernel */
     CWICK_HIP_PROF_GQA_DECODE_MERGE,    /* splitk_merge_wide_kernel<256|128> after it */
     CWICK_HIP_PROF_GQA_PREFILL,         /* gqa_prefill_kernel */
-    CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill of at most 64 heads) */
+    CWICK_HIP_PROF_MLA,                 /* mla_roles_kernel (decode, sparse, prefill of at most 32 heads) */
     CWICK_HIP_PROF_MLA_MERGE,           /* mla_merge_frag16_kernel after it */
     CWICK_HIP_PROF_INDEXER,             /* indexer_scores_kernel, or in a fused select indexer_approx_kernel + topk_mw_hist_kernel + topk_mw_classify_kernel + indexer_rescore_kernel + the exact kernel's fallback pass */
     CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel; in a fused select topk_band_finish_kernel */
-    CWICK_HIP_PROF_MLA_PREFILL,         /* mla_prefill64_kernel (chunked prefill of more than 64 heads) */
+    CWICK_HIP_PROF_MLA_PREFILL,         /* mla_prefill64_kernel (chunked prefill of more than 32 heads) */
     CWICK_HIP_PROF_MM_SELECT,           /* mm_index_scores[_long]_kernel + mm_pick_kernel; for block sizes that are not a multiple of 64 mm_blockmax_kernel and mm_expand_kernel, with the block top-k between them under CWICK_HIP_PROF_TOPK */
     CWICK_HIP_PROF_COUNT
 };

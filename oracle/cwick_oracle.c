@@ -1139,23 +1139,6 @@ ORC_API int orc_mm_select_blocks(const float *scores, int64_t limit, int bs, int
     return nb;
 }
 
-/* ------------------------------------------------------------------ */
-/* DSA decode = indexer -> top-k -> sparse MLA (BASELINE config 5)     */
-/* ------------------------------------------------------------------ */
-ORC_API void orc_dsa_decode(const uint16_t *qidx_bf16, const float *w,
-                            const uint8_t *ikeys, const float *ikscale,
-                            int64_t n_keys, int ih, int ihd, int64_t topk,
-                            const uint16_t *q_bf16, const uint8_t *lat,
-                            const float *lat_scales, int64_t kdim, int64_t vdim,
-                            int64_t block, int nh, float scale, int nthreads,
-                            float *scores_tmp /* [n_keys] */,
-                            int32_t *sel_out /* [topk] */, float *out) {
-    orc_indexer_scores(qidx_bf16, w, ikeys, ikscale, n_keys, ih, ihd, nthreads, scores_tmp);
-    int64_t got = orc_topk_contract(scores_tmp, n_keys, topk, sel_out);
-    orc_mla_decode(q_bf16, lat, lat_scales, kdim, vdim, block, sel_out, got, nh,
-                   scale, nthreads, out);
-}
-
 /* src/prof.c:39-43 (cwick_prof_ns): CLOCK_MONOTONIC in nanoseconds. */
 ORC_API int64_t orc_now_ns(void) {
     struct timespec ts;

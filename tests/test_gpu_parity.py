@@ -451,6 +451,33 @@ def test_dsa_select_ties_at_the_threshold(hip, orc, n_keys, topk, copies, take, 
         say("[parity] query %d: %d keys tie at the threshold, %d of them selected" % (b, tied, inside))
         assert tied >= copies and inside < tied or take == copies
         assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
+        ref = orc.mla_decode(c["q"][b], c["rows"][b], c["scales"][b], c["scale"], sel=rsel, nthreads=0)
+        assert_close(out[b], ref, "dsa_decode with ties, query %d of %d" % (b, batch))
+    ik.free()
+    lat.free()
+
+
+def test_dsa_decode_as_benchmarked(hip, orc):
+    """BASELINE config 5 exactly as bench.py times it: eight independent queries with caches of
+    their own, 65536 keys, 64 index heads, top-2048, 128 heads.  The batch sets the number of key
+    slices per query (and with it the merge path), so this is not the batch-3 case above: selected
+    rows bit for bit and the outputs of all eight queries."""
+    say("[case] dsa_decode as benchmarked: batch 8, 65536 keys, top-2048")
+    c = synth.cfg5_dsa()
+    B, N, K = c["batch"], c["n_keys"], c["topk"]
+    assert (B, N, K, c["ih"], c["nh"]) == (8, 65536, 2048, 64, 128)
+    ik = hip.IndexKeys(B, N)
+    lat = hip.LatentCache(B, N)
+    for b in range(B):
+        ik.write(b, 0, c["ikeys"][b], c["ikscale"][b])
+        lat.write(b, 0, c["rows"][b], c["scales"][b])
+    out, sel = hip.dsa_decode(ik, lat, 0, 1, N, c["q_idx"], c["w"], K, c["q"], c["scale"])
+    for b in range(B):
+        sc = orc.indexer_scores(c["q_idx"][b], c["w"][b], c["ikeys"][b], c["ikscale"][b], nthreads=0)
+        rsel = orc.topk_contract(sc, K)
+        assert np.array_equal(sel[b], rsel), "query %d: selected rows differ" % b
+        ref = orc.mla_decode(c["q"][b], c["rows"][b], c["scales"][b], c["scale"], sel=rsel, nthreads=0)
+        assert_close(out[b], ref, "dsa_decode as benchmarked, query %d" % b)
     ik.free()
     lat.free()
 
@@ -782,6 +809,63 @@ def test_mla_decode_sink(hip, orc, n_rows, n_sel):
     cache.free()
 
 
+@pytest.mark.parametrize("pos,W,n_cmp,topk", [(50, 128, 0, 64), (127, 128, 31, 64), (1000, 128, 250, 64),
+                                              (5000, 128, 1250, 512)])
+def test_window_ring_and_compressed_rows_with_sink(hip, orc, pos, W, n_cmp, topk):
+    """ds_sparse_attn_heads' key list (src/ds_model.c:917-932, built at :1214-1237): a ring of W
+    window rows written at slot pos % W, then the compressed rows; idx[] holds the ring slots of
+    the W positions ending at pos (oldest first, -1 where the sequence has not got to), then W + j
+    for the compressed rows the indexer kept (-1 padded).  With the store laid out
+    [ring | compressed] idx[] is a row list as it stands: the sparse decode with the sink against
+    the oracle over a host mirror of the same store."""
+    say("[case] window ring + compressed rows + sink", pos, W, n_cmp, topk)
+    nh = 128
+    g = synth.rng(8800 + pos)
+    n_pos = pos + 1
+    lat_rows, lat_scales = synth.latent_cache(g, n_pos)             # the window latent of every position so far
+    cmp_rows, cmp_scales = synth.latent_cache(g, max(n_cmp, 1))
+    q = synth.normal_bf16(g, (nh, synth.KDIM))
+    scale = float(1.0 / np.sqrt(192.0))
+    cache = hip.LatentCache(1, W + max(n_cmp, 1))
+    ring_rows = np.zeros((W, synth.KDIM), np.uint8)
+    ring_scales = np.zeros((W, synth.NBLK), np.float32)
+    cache.write(0, 0, ring_rows, ring_scales)                        # the reference clears the ring (:714)
+    # written in wrap order, one position at a time where the ring wraps (the last 2 W positions),
+    # so that slots are overwritten on the device as the engine would
+    first_single = max(0, n_pos - 2 * W)
+    for pp in range(first_single):
+        ring_rows[pp % W] = lat_rows[pp]; ring_scales[pp % W] = lat_scales[pp]
+    if first_single:
+        cache.write(0, 0, ring_rows, ring_scales)
+    for pp in range(first_single, n_pos):
+        ring_rows[pp % W] = lat_rows[pp]; ring_scales[pp % W] = lat_scales[pp]
+        cache.write(0, pp % W, lat_rows[pp:pp + 1], lat_scales[pp:pp + 1])
+    if n_cmp:
+        cache.write(0, W, cmp_rows, cmp_scales)
+    idx = []
+    lo = max(0, pos - W + 1)
+    for pp in range(lo, pos + 1):
+        idx.append(pp % W)
+    idx += [-1] * (W - len(idx))
+    ncmp = min(n_cmp, topk)
+    kept = np.sort(g.permutation(n_cmp)[:ncmp]) if n_cmp else np.zeros(0, np.int64)
+    idx += [W + int(j) for j in kept]
+    idx = np.array(idx, np.int32)
+    assert idx.size == W + ncmp
+    sink = (g.standard_normal(nh) * 2.0 + 4.0).astype(np.float32)
+    store_rows = np.concatenate([ring_rows, cmp_rows]); store_scales = np.concatenate([ring_scales, cmp_scales])
+    got = hip.mla_decode(cache, 0, q, scale, sel=idx, sink=sink)
+    ref = orc.sparse_attn_sink(q, store_rows, store_scales, scale, sink=sink, sel=idx, nthreads=0)
+    assert_close(got, ref, "window ring pos %d" % pos)
+    # the ring really holds the last W positions: the same output from a list over the positions' own latents
+    live = np.arange(lo, pos + 1)
+    flat_rows = np.concatenate([lat_rows[live], cmp_rows[kept]]) if ncmp else lat_rows[live]
+    flat_scales = np.concatenate([lat_scales[live], cmp_scales[kept]]) if ncmp else lat_scales[live]
+    ref2 = orc.sparse_attn_sink(q, flat_rows, flat_scales, scale, sink=sink, sel=None, nthreads=0)
+    assert np.abs(ref - ref2).max() <= 1e-5 * max(1.0, np.abs(ref2).max())
+    cache.free()
+
+
 # ------------------------------------------------------------------ the DeepSeek indexer flavour
 @pytest.mark.parametrize("n_keys,ih", [(65536, 64), (1000, 32), (257, 7), (1, 64)])
 def test_indexer_scores_ds_mode_bit_exact(hip, orc, n_keys, ih):
@@ -958,7 +1042,10 @@ def test_ikeys_pool_append_on_device(hip, orc, kp, n_pools):
 
 
 @pytest.mark.parametrize("batch,n,bs,keep", [(1, 65536, 64, 32), (4, 10000, 128, 8), (2, 65, 64, 1), (3, 300, 7, 50),
-                                             (1, 5, 64, 3), (2, 131072, 64, 512)])
+                                             (1, 5, 64, 3), (2, 131072, 64, 512),
+                                             # more than 14336 blocks: the block top-k is the many-workgroup select,
+                                             # which keeps a workspace of its own next to this call's block scores
+                                             (1, 16000, 1, 100), (2, 31000, 2, 64)])
 def test_candidate_blocks_on_device(hip, orc, batch, n, bs, keep):
     """Level one of the two-level selection (src/ds_model.c:1125-1148): the byte mask bit for bit
     against the oracle's, then masked scores -> top-k equal to the oracle's selection over its own
@@ -1107,6 +1194,8 @@ def test_gqa_decode_over_selected_blocks(hip, orc, n_rows, nh, nkv, hd, bs, keep
     (300, 1, 2, 512, 128, 16, 4096),       # more blocks asked for than exist
     (70000, 1, 4, 128, 64, 16, 4096),      # more than 1024 blocks: the streaming row select inside the one-workgroup step
     (9000, 3, 4, 128, 192, 5, 4096),       # blocks of three scoring groups
+    (45000, 2, 2, 64, 3, 16, 4096),        # 15000 blocks of a size the scoring groups do not divide: block maxima,
+                                           # the many-workgroup top-k (its own workspace), expansion
 ])
 def test_mm_select_blocks_on_device(hip, orc, limit0, batch, ih, idim, bs, keep, max_sel):
     """The block selection of the block-sparse decode (src/mm_model.c:1764-1780, :1733-1761,
