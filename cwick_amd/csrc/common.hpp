@@ -1,6 +1,7 @@
 // common.hpp -- shared declarations of libcwick_hip.so (gfx950 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stddef.h>
 
@@ -48,6 +49,29 @@ struct ProfScope {
     int which;
     hipStream_t stream;
     void *slot;
+};
+
+// Phase timer of exactly one kernel: when profiling is enabled the launch goes through
+// hipExtLaunchKernelGGL with a start and a stop event that the runtime binds to the dispatch
+// itself, so their difference is the kernel's own duration (what a kernel trace reports), not
+// the dispatch latency that an event pair recorded around the launch includes.  Otherwise an
+// ordinary launch, no events.
+struct ProfKernel {
+    ProfKernel(int which, hipStream_t s);
+    ~ProfKernel();
+    template <typename... KArgs, typename... Args>
+    void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t smem, Args... args) {
+        if (a) {
+            hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)smem, stream, a, b, 0u, static_cast<KArgs>(args)...);
+            bound = true;
+        } else {
+            kernel<<<grid, block, smem, stream>>>(static_cast<KArgs>(args)...);
+        }
+    }
+    int which;
+    hipStream_t stream;
+    hipEvent_t a = nullptr, b = nullptr;
+    bool bound = false;
 };
 
 // ---- kernel launchers (one per .hip file) ----------------------------------

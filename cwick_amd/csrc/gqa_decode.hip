@@ -260,15 +260,15 @@ static int run_gqa_decode(const uint16_t *k, const uint16_t *v, int64_t n_keys, 
     if (!ws) return 0;                      // workspace() has recorded why
     float *part_acc = (float *)ws, *part_ml = (float *)(ws + acc_bytes);
     {
-        ProfScope ps(CWICK_HIP_PROF_GQA_DECODE, s);
-        gqa_decode_split_kernel<HD, GROUP><<<dim3(n_splits, n_units), GQA_DEC_THREADS, 0, s>>>(
-            k, v, q, n_keys, n_kv_heads, sel, n_rows, (int)per, kv_shift, scale, part_acc, part_ml);
+        ProfKernel pk(CWICK_HIP_PROF_GQA_DECODE, s);
+        pk.launch(gqa_decode_split_kernel<HD, GROUP>, dim3(n_splits, n_units), dim3(GQA_DEC_THREADS), 0,
+                  k, v, q, n_keys, n_kv_heads, sel, n_rows, (int)per, kv_shift, scale, part_acc, part_ml);
     }
     CWICK_HIP_CALL(hipGetLastError());
     {
-        ProfScope ps(CWICK_HIP_PROF_GQA_DECODE_MERGE, s);
-        splitk_merge_wide_kernel<HD><<<dim3(n_heads, 1), 64 * (n_splits < 16 ? n_splits : 16), 0, s>>>(
-            part_acc, part_ml, n_splits, n_heads, out);
+        ProfKernel pk(CWICK_HIP_PROF_GQA_DECODE_MERGE, s);
+        pk.launch(splitk_merge_wide_kernel<HD>, dim3(n_heads, 1), dim3(64 * (n_splits < 16 ? n_splits : 16)), 0,
+                  part_acc, part_ml, n_splits, n_heads, out);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

@@ -758,9 +758,9 @@ static int run_gqa_prefill(const uint16_t *k, const uint16_t *v, int64_t pos0, i
     const int64_t items = pblocks * n_kv_heads;
     const int64_t wgs = items < num_cus() ? items : num_cus();      // the LDS of a compute unit holds one workgroup
     {
-        ProfScope ps(CWICK_HIP_PROF_GQA_PREFILL, s);
-        gqa_prefill_kernel<GROUP><<<dim3((unsigned)wgs), PF_THREADS, smem, s>>>(
-            k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec, pblocks, tickets);
+        ProfKernel pk(CWICK_HIP_PROF_GQA_PREFILL, s);
+        pk.launch(gqa_prefill_kernel<GROUP>, dim3((unsigned)wgs), dim3(PF_THREADS), smem,
+                  k, v, q, pos0, n, n_kv_heads, scale * 1.44269504088896340736f, out, n_prec, pblocks, tickets);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

@@ -409,9 +409,12 @@ int launch_indexer_approx(const uint8_t *keys, const float *kscale, int64_t key_
     CWICK_REQUIRE((uintptr_t)keys % 16 == 0 && key_bstride % 16 == 0 && (uintptr_t)q_idx % 16 == 0,
                   "indexer_approx: keys and q must be 16-byte aligned");
     const int n_wg = indexer_approx_slots(n_keys);
-    indexer_approx_kernel<<<dim3(n_wg, batch), IB_THREADS, 0, s>>>(
-        keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows,
-        digit0_slices, digit0_row_dwords);
+    {
+        ProfKernel pk(CWICK_HIP_PROF_INDEXER_APPROX, s);
+        pk.launch(indexer_approx_kernel, dim3(n_wg, batch), dim3(IB_THREADS), 0,
+                  keys, kscale, key_bstride, kscale_bstride, n_keys, q_idx, w, n_idx_heads, scores, beta_slots, rows,
+                  digit0_slices, digit0_row_dwords);
+    }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;
 }

@@ -582,8 +582,8 @@ int launch_mla_prefill_wide(const uint8_t *rows, const float *scales, int64_t po
     const int64_t total = (int64_t)n_hb * n;
     CWICK_REQUIRE(total <= 0x7FFFFFFF, "mla_prefill: grid of %lld workgroups is too large", (long long)total);
     {
-        ProfScope ps(CWICK_HIP_PROF_MLA_PREFILL, s);
-        mla_prefill64_kernel<<<dim3((unsigned)total), THREADS, smem, s>>>(p);
+        ProfKernel pk(CWICK_HIP_PROF_MLA_PREFILL, s);
+        pk.launch(mla_prefill64_kernel, dim3((unsigned)total), dim3(THREADS), smem, p);
     }
     CWICK_HIP_CALL(hipGetLastError());
     return 1;

@@ -962,19 +962,19 @@ int run(Params &p, hipStream_t s, bool fixed = false) {
         p.part_ml = (float *)(ws + acc_b);
     }
     {
-        ProfScope ps(fixed ? -1 : CWICK_HIP_PROF_MLA, s);
-        if (p.sel) mla_roles_kernel<true><<<dim3((unsigned)total), THREADS, smem, s>>>(p);
-        else mla_roles_kernel<false><<<dim3((unsigned)total), THREADS, smem, s>>>(p);
+        ProfKernel pk(fixed ? -1 : CWICK_HIP_PROF_MLA, s);
+        if (p.sel) pk.launch(mla_roles_kernel<true>, dim3((unsigned)total), dim3(THREADS), smem, p);
+        else pk.launch(mla_roles_kernel<false>, dim3((unsigned)total), dim3(THREADS), smem, p);
     }
     CWICK_HIP_CALL(hipGetLastError());
     if (p.n_splits > 1) {
-        ProfScope ps(fixed ? -1 : CWICK_HIP_PROF_MLA_MERGE, s);
+        ProfKernel pk(fixed ? -1 : CWICK_HIP_PROF_MLA_MERGE, s);
         if (p.n_splits <= 8)
-            mla_merge_frag16_kernel<<<dim3(2 * n_hb * 4, p.nq), 64 * 8, 0, s>>>(
-                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 1);
+            pk.launch(mla_merge_frag16_kernel, dim3(2 * n_hb * 4, p.nq), dim3(64 * 8), 0, p.part_acc, p.part_ml,
+                      p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 1);
         else
-            mla_merge_frag16_kernel<<<dim3(2 * n_hb * NDB, p.nq), 64 * (p.n_splits <= 64 ? 8 : MW), 0, s>>>(
-                p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 0);
+            pk.launch(mla_merge_frag16_kernel, dim3(2 * n_hb * NDB, p.nq), dim3(64 * (p.n_splits <= 64 ? 8 : MW)), 0,
+                      p.part_acc, p.part_ml, p.n_splits, 2 * n_hb, p.nh, p.sink, p.out, 0);
         CWICK_HIP_CALL(hipGetLastError());
     }
     return 1;

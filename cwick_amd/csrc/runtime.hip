@@ -251,6 +251,29 @@ ProfScope::~ProfScope() {
     delete pp;
 }
 
+ProfKernel::ProfKernel(int w, hipStream_t s) : which(w), stream(s) {
+    if (!g_prof_on || w < 0) return;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfPair pp;
+    if (!g_prof_free.empty()) {
+        pp = g_prof_free.back();
+        g_prof_free.pop_back();
+    } else if (hipEventCreate(&pp.a) != hipSuccess || hipEventCreate(&pp.b) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    a = pp.a;
+    b = pp.b;
+}
+
+ProfKernel::~ProfKernel() {
+    if (!a) return;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfPair pp{a, b, which};
+    if (bound) g_prof_pending.push_back(pp);
+    else g_prof_free.push_back(pp);
+}
+
 static void prof_drain_locked() {
     for (ProfPair &pp : g_prof_pending) {
         float ms = 0.0f;
@@ -1126,7 +1149,7 @@ const char *cwick_hip_prof_name(int which) {
     static const char *names[CWICK_HIP_PROF_COUNT] = {
         "gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
         "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel",
-        "mm select kernels"};
+        "mm select kernels", "indexer_approx_kernel"};
     return which >= 0 && which < CWICK_HIP_PROF_COUNT ? names[which] : "";
 }
 

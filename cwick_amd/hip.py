@@ -609,7 +609,7 @@ def candidate_apply_dev(scores, cand, batch, n, stream=None):
 # ------------------------------------------------------------------ phase timers
 PROF_NAMES = ["gqa_decode_split_kernel", "splitk_merge_wide_kernel<gqa>", "gqa_prefill_kernel",
               "mla_roles_kernel", "mla_merge_frag16_kernel", "indexer kernels", "topk kernels", "mla_prefill64_kernel",
-              "mm select kernels"]
+              "mm select kernels", "indexer_approx_kernel"]
 
 
 def prof_enable(on=True):

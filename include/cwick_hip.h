@@ -491,11 +491,14 @@ int cwick_hip_ikeys_read_f32(cwick_hip_ikeys *c, int slot, int64_t pos0, int64_t
 /* ---- phase timers ------------------------------------------------------- */
 /* Replace the reference's attention sub-timers (g_attn_*_ns, src/attention.c:1169-1174,
  * read out by src/prof.c:184-196 under CWICK_PROFILE; CWICK_Q35_PROF's
- * qk/softmax/av split, src/q35_model.c:72-99).  While enabled, every launch of
- * a kernel listed below is bracketed by a pair of HIP events on the stream it
- * is launched on; cwick_hip_prof_read() waits for the recorded events and
- * returns the summed GPU time and the number of launches since the last reset.
- * Off by default (no events are recorded). */
+ * qk/softmax/av split, src/q35_model.c:72-99).  While enabled, an entry that
+ * names one kernel is timed by a start and a stop event bound to that kernel's
+ * dispatch (hipExtLaunchKernel): the kernel's own duration, as a kernel trace
+ * reports it.  An entry that names several kernels is bracketed by a pair of
+ * events recorded on the stream around the launches, which also counts the
+ * dispatch latency between them.  cwick_hip_prof_read() waits for the
+ * recorded events and returns the summed GPU time and the number of timed
+ * sections since the last reset.  Off by default (no events are recorded). */
 enum {
     CWICK_HIP_PROF_GQA_DECODE = 0,      /* gqa_decode_split_kernel */
     CWICK_HIP_PROF_GQA_DECODE_MERGE,    /* splitk_merge_wide_kernel<256|128> after it */
@@ -506,6 +509,7 @@ enum {
     CWICK_HIP_PROF_TOPK,                /* every kernel of one top-k call: topk_mw_hist_kernel x4 + topk_mw_emit_kernel, or topk_radix[_reg]_kernel; in a fused select topk_band_finish_kernel */
     CWICK_HIP_PROF_MLA_PREFILL,         /* mla_prefill64_kernel (chunked prefill of more than 32 heads) */
     CWICK_HIP_PROF_MM_SELECT,           /* mm_index_scores[_long]_kernel + mm_pick_kernel; for block sizes that are not a multiple of 64 mm_blockmax_kernel and mm_expand_kernel, with the block top-k between them under CWICK_HIP_PROF_TOPK */
+    CWICK_HIP_PROF_INDEXER_APPROX,      /* indexer_approx_kernel alone (also counted inside CWICK_HIP_PROF_INDEXER) */
     CWICK_HIP_PROF_COUNT
 };
 void cwick_hip_prof_enable(int on);
