@@ -166,6 +166,8 @@ int launch_mm_select(const uint16_t *idx_keys, const float *iq, int batch, int64
                      int index_dim, int block, int keep_blocks, float *scores, int64_t score_stride,
                      int32_t *blk_out, int32_t *sel, int64_t max_sel, int32_t *n_sel, hipStream_t s);
 int launch_candidate_apply(float *scores, const uint8_t *cand, int batch, int64_t n, hipStream_t s);
+int launch_glm_select(const float *scores, int batch, int64_t n_comp, int64_t npos, int kpool, int64_t topk,
+                      int strict, int32_t *sel, int64_t max_sel, int32_t *n_sel, hipStream_t s);
 int launch_dequant_latent(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
 int launch_dequant_ikeys(const uint8_t *rows, const float *scales, int64_t n, float *out, hipStream_t s);
 int launch_widen_bf16(const uint16_t *src, int64_t n, float *dst, hipStream_t s);

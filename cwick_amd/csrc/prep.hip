@@ -373,6 +373,131 @@ int launch_candidate_select(const float *scores, int batch, int64_t n, int block
     return 1;
 }
 
+// The rest of indexer_select behind the pool scores (src/attention.c:585-620), one workgroup per
+// query.  pools[want] are the chosen pools in ascending order (the top-k select's output);
+// the list keeps the reference's order: the pools that score above the lowest chosen score in
+// ascending order, then the pools that equal it, each as its kp positions c kp + r; the
+// positions behind the last closed pool; then the query's own position unless `strict` or it is
+// the last entry already (the reference tests sel[n-1] only, :618).  mode_whole: no more pools
+// than wanted -- the list is the whole prefix 0 .. npos-1 and n_sel is -1 (:558-559).
+// Entries behind the list are -1, which the attention kernels skip.
+constexpr int GLM_THREADS = 256;
+__global__ void __launch_bounds__(GLM_THREADS)
+glm_expand_kernel(const float *__restrict__ scores, const int32_t *__restrict__ pools, int64_t want, int64_t n_comp,
+                  int64_t npos, int kp, int strict, int mode_whole, int32_t *__restrict__ sel, int64_t max_sel,
+                  int32_t *__restrict__ n_sel) {
+    __shared__ uint32_t red[GLM_THREADS / 64];
+    __shared__ uint32_t wave_gt[GLM_THREADS / 64], wave_eq[GLM_THREADS / 64];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int32_t *out = sel + (size_t)row * max_sel;
+    if (mode_whole) {
+        for (int64_t i = tid; i < max_sel; i += GLM_THREADS) out[i] = i < npos ? (int32_t)i : -1;
+        if (tid == 0 && n_sel) n_sel[row] = -1;
+        return;
+    }
+    const float *sc = scores + (size_t)row * n_comp;
+    const int32_t *pl = pools + (size_t)row * want;
+    // the lowest chosen score, as the select's own order key (so that -0.0 == +0.0)
+    uint32_t kmin = 0xFFFFFFFFu;
+    for (int64_t i = tid; i < want; i += GLM_THREADS) {
+        const int32_t c = pl[i];
+        if (c >= 0) {
+            const uint32_t k = topk_key(sc[c]);
+            kmin = k < kmin ? k : kmin;
+        }
+    }
+    kmin = wave_min_u32(kmin);
+    if (lane == 0) red[wave] = kmin;
+    __syncthreads();
+    kmin = red[0];
+#pragma unroll
+    for (int w = 1; w < GLM_THREADS / 64; w++) kmin = red[w] < kmin ? red[w] : kmin;
+    // how many chosen pools score above it (they come first), and the last pool at it (the list's
+    // last pool entry)
+    uint32_t n_gt = 0, eq_last = 0;                 // eq_last: pool index + 1
+    for (int64_t i = tid; i < want; i += GLM_THREADS) {
+        const int32_t c = pl[i];
+        if (c < 0) continue;
+        if (topk_key(sc[c]) > kmin) n_gt++;
+        else eq_last = (uint32_t)c + 1u > eq_last ? (uint32_t)c + 1u : eq_last;
+    }
+    n_gt = wave_sum_u32(n_gt);
+    eq_last = wave_max_u32(eq_last);
+    __syncthreads();
+    if (lane == 0) red[wave] = n_gt, wave_eq[wave] = eq_last;
+    __syncthreads();
+    n_gt = 0, eq_last = 0;
+#pragma unroll
+    for (int w = 0; w < GLM_THREADS / 64; w++) {
+        n_gt += red[w];
+        eq_last = wave_eq[w] > eq_last ? wave_eq[w] : eq_last;
+    }
+    // places: a running count of both kinds over chunks of the pool list
+    uint32_t base_gt = 0, base_eq = 0;
+    for (int64_t i0 = 0; i0 < want; i0 += GLM_THREADS) {
+        const int64_t i = i0 + tid;
+        const int32_t c = i < want ? pl[i] : -1;
+        const bool gt = c >= 0 && topk_key(sc[c]) > kmin, eq = c >= 0 && !gt;
+        const uint32_t sg = wave_scan_u32(gt ? 1u : 0u), se = wave_scan_u32(eq ? 1u : 0u);
+        __syncthreads();
+        if (lane == 63) wave_gt[wave] = sg, wave_eq[wave] = se;
+        __syncthreads();
+        uint32_t og = base_gt, oe = base_eq, tg = 0, te = 0;
+#pragma unroll
+        for (int w = 0; w < GLM_THREADS / 64; w++) {
+            if (w < wave) og += wave_gt[w], oe += wave_eq[w];
+            tg += wave_gt[w], te += wave_eq[w];
+        }
+        if (c >= 0) {
+            const uint32_t place = gt ? og + sg - 1u : n_gt + oe + se - 1u;
+            for (int r = 0; r < kp; r++) out[(size_t)place * kp + r] = c * kp + r;
+        }
+        base_gt += tg, base_eq += te;
+    }
+    __syncthreads();
+    // the tail, the query itself, the padding: one thread (a handful of entries) and then all
+    const int64_t n_pool = (int64_t)(base_gt + base_eq) * kp;
+    const int64_t tail = npos % kp;
+    int64_t n = n_pool + tail;
+    for (int64_t r = tid; r < tail; r += GLM_THREADS) out[n_pool + r] = (int32_t)(npos - tail + r);
+    // the list's last entry before the self rule: the tail's, else the last pool at the lowest score
+    const int64_t last = tail > 0 ? npos - 1 : (eq_last ? (int64_t)(eq_last - 1u) * kp + kp - 1 : -1);
+    const bool add_self = !strict && last != npos - 1;
+    if (tid == 0 && add_self) out[n] = (int32_t)(npos - 1);
+    if (add_self) n++;
+    for (int64_t i = n + tid; i < max_sel; i += GLM_THREADS) out[i] = -1;
+    if (tid == 0 && n_sel) n_sel[row] = (int32_t)n;
+}
+
+int launch_glm_select(const float *scores, int batch, int64_t n_comp, int64_t npos, int kpool, int64_t topk,
+                      int strict, int32_t *sel, int64_t max_sel, int32_t *n_sel, hipStream_t s) {
+    CWICK_REQUIRE(scores && sel, "glm_select: null pointer");
+    CWICK_REQUIRE(batch >= 1 && batch <= 65535 && n_comp >= 1 && n_comp <= ((int64_t)1 << 24),
+                  "glm_select: batch %d, %lld pools", batch, (long long)n_comp);
+    CWICK_REQUIRE(kpool >= 1 && kpool <= 8, "glm_select: kpool %d (1..8, src/attention.c:492)", kpool);
+    CWICK_REQUIRE(topk >= 1 && topk <= 65536, "glm_select: topk %lld", (long long)topk);
+    CWICK_REQUIRE(npos >= n_comp * kpool && npos < (n_comp + 1) * kpool,
+                  "glm_select: %lld positions do not close exactly %lld pools of %d", (long long)npos,
+                  (long long)n_comp, kpool);
+    const int64_t want = (topk + kpool - 1) / kpool;
+    CWICK_REQUIRE(max_sel >= (want + 1) * kpool && max_sel <= ((int64_t)1 << 24),
+                  "glm_select: max_sel %lld (at least (ceil(topk / kpool) + 1) * kpool = %lld)", (long long)max_sel,
+                  (long long)((want + 1) * kpool));
+    if (n_comp <= want) {
+        glm_expand_kernel<<<dim3(batch), GLM_THREADS, 0, s>>>(scores, nullptr, want, n_comp, npos, kpool, strict, 1, sel,
+                                                            max_sel, n_sel);
+        CWICK_HIP_CALL(hipGetLastError());
+        return 1;
+    }
+    int32_t *pools = (int32_t *)workspace(s, (size_t)batch * want * sizeof(int32_t));
+    if (!pools) return 0;                   // workspace() has recorded why
+    if (!launch_topk(scores, batch, n_comp, want, pools, s)) return 0;
+    glm_expand_kernel<<<dim3(batch), GLM_THREADS, 0, s>>>(scores, pools, want, n_comp, npos, kpool, strict, 0, sel,
+                                                        max_sel, n_sel);
+    CWICK_HIP_CALL(hipGetLastError());
+    return 1;
+}
+
 int launch_candidate_apply(float *scores, const uint8_t *cand, int batch, int64_t n, hipStream_t s) {
     CWICK_REQUIRE(scores && cand && batch >= 1 && n >= 1, "candidate_apply: bad argument");
     const int64_t total = (int64_t)batch * n;

@@ -1211,6 +1211,13 @@ int cwick_hip_candidate_apply_dev(float *scores, const uint8_t *cand, int batch,
     return launch_candidate_apply(scores, cand, batch, n, (hipStream_t)stream);
 }
 
+int cwick_hip_glm_select_dev(const float *scores, int batch, int64_t n_comp, int64_t npos, int kpool, int64_t topk,
+                             int strict, int32_t *sel, int64_t max_sel, int32_t *n_sel, void *stream) {
+    clear_error();
+    if (!backend_ready()) return 0;   /* the reason is recorded */
+    return launch_glm_select(scores, batch, n_comp, npos, kpool, topk, strict, sel, max_sel, n_sel, (hipStream_t)stream);
+}
+
 int cwick_hip_mm_select_dev(const uint16_t *idx_keys, const float *iq, int batch, int64_t limit0, int index_heads,
                             int index_dim, int block, int keep_blocks, float *scores, int64_t score_stride,
                             int32_t *blk_out, int32_t *sel, int64_t max_sel, int32_t *n_sel, void *stream) {

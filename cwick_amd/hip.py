@@ -94,6 +94,7 @@ SIGNATURES = {
     "cwick_hip_ikeys_pool_append_dev": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _flt, _int, _vp, _vp]),
     "cwick_hip_candidate_select_dev": (_int, [_vp, _int, _i64, _int, _i64, _vp, _vp]),
     "cwick_hip_candidate_apply_dev": (_int, [_vp, _vp, _int, _i64, _vp]),
+    "cwick_hip_glm_select_dev": (_int, [_vp, _int, _i64, _i64, _int, _i64, _int, _vp, _i64, _vp, _vp]),
     "cwick_hip_mm_select": (_int, [_vp, _i64, _vp, _int, _int, _int, _vp, _vp, _i64, _vp]),
     "cwick_hip_mm_select_dev": (_int, [_vp, _vp, _int, _i64, _int, _int, _int, _int, _vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "cwick_hip_latent_read_f32": (_int, [_vp, _int, _i64, _i64, _vp]),
@@ -599,6 +600,12 @@ def workspace_bytes_dev(stream):
 def stream_release(stream, raw=False):
     rc = lib().cwick_hip_stream_release(stream)
     return rc if raw else _check(rc, "stream_release")
+
+
+def glm_select_dev(scores, batch, n_comp, npos, kpool, topk, strict, sel, max_sel, n_sel, stream=None, raw=False):
+    rc = lib().cwick_hip_glm_select_dev(_dp(scores), batch, n_comp, npos, kpool, topk, 1 if strict else 0, _dp(sel),
+                                        max_sel, _dp(n_sel), stream)
+    return rc if raw else _check(rc, "glm_select_dev")
 
 
 def candidate_apply_dev(scores, cand, batch, n, stream=None):

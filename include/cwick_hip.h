@@ -459,6 +459,31 @@ int cwick_hip_ikeys_pool_append_dev(cwick_hip_ikeys *c, int slot, int64_t pos0, 
                                     const float *k_norm_b, float eps, int kpool,
                                     float *rows_f32, void *stream);
 
+/* Replaces the rest of indexer_select behind the pool scores (src/attention.c:
+ * 585-620), so that a chain indexer scores -> selection -> sparse attention
+ * with index_kpool > 1 stays on the device.  scores fp32 [batch][n_comp], one
+ * per closed pool of `kpool` positions (what cwick_hip_indexer_scores_dev
+ * leaves); every query of the batch stands at position npos - 1, with
+ * n_comp = npos / kpool.  want = ceil(topk / kpool) pools are kept: the best
+ * by (score descending, pool index ascending), i.e. the reference's
+ * `> thr` then `== thr` passes with thr the want-th largest score (its
+ * quickselect can leave a larger threshold and then takes fewer pools,
+ * src/attention.c:529-543 and :590; this call always takes `want`).  The
+ * list sel[batch][max_sel] is in the reference's order: the pools above the
+ * threshold ascending, then the pools at it, each as positions c*kpool + r
+ * (:592-598); the npos % kpool positions behind the last closed pool
+ * (:603-604); and, unless `strict` (CWICK_INDEXER_STRICT), npos - 1 when the
+ * list does not already END with it (:618-620 tests the last entry only, so a
+ * selected last pool that is not the threshold pool is followed by a second
+ * copy of npos - 1, as in the reference).  Entries behind the list are -1;
+ * n_sel[batch] (may be NULL) receives the count.  When n_comp <= want the
+ * reference attends to the whole prefix (:558-559): the list is then
+ * 0 .. npos-1 and n_sel is -1.  max_sel >= (want + 1) * kpool; pass sel with
+ * n_list = max_sel to cwick_hip_mla_decode_dev, which skips the -1 entries. */
+int cwick_hip_glm_select_dev(const float *scores, int batch, int64_t n_comp, int64_t npos,
+                             int kpool, int64_t topk, int strict, int32_t *sel, int64_t max_sel,
+                             int32_t *n_sel, void *stream);
+
 /* Replaces level one of the two-level selection on the layer that is the
  * candidate source (src/ds_model.c:1125-1144): the maximum score of every
  * block of `block` positions, the last (partly filled) block forced in with

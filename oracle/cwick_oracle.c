@@ -39,6 +39,12 @@
  *                                      separate the threshold at want-1 from want and
  *                                      show the under-selection), subset-of-contract
  *                                      property
+ *   orc_glm_select                     known answers traced by hand through
+ *                                      src/attention.c:585-620 (tail present and absent, the
+ *                                      query kept already / pruned / repeated, the strict flag,
+ *                                      no more pools than wanted), on the score vectors of the
+ *                                      quickselect traces; the contract's pool choice against the
+ *                                      reference's where the two agree and where they do not
  *   orc_gqa_decode / orc_gqa_prefill   double brute force, decode==prefill row,
  *                                      rectangle==triangle: PARITY UNPINNED against a
  *                                      reference build, pinned by mathematics only
@@ -1012,6 +1018,54 @@ ORC_API int64_t orc_topk_quickselect(const float *sc, int64_t n, int64_t want, i
         }
     free(cp);
     return m;
+}
+
+/* src/attention.c:548-622 after the scores (:585-620): which positions a query keeps.  `sc` holds
+ * one score per closed pool (n_comp = npos / kp of them).  want = ceil(topk / kp) pools; when there
+ * are no more pools than that the answer is "the whole prefix" (-1, :558-559).  Otherwise the pools
+ * are chosen, each expands to its kp positions c kp + r (:592-598), the positions behind the last
+ * closed pool are always kept (:603-604), and unless `strict` (CWICK_INDEXER_STRICT, :618-620) the
+ * query's own position npos - 1 is added when it is not the last entry already.
+ * The list keeps the reference's order: the pools above the threshold in ascending order, then
+ * the pools that equal it, then the tail, then the query itself -- whose test looks at the last
+ * entry only (:618), so a last pool that was selected above the threshold is followed by a second
+ * copy of npos - 1; that is the reference's behaviour and it is kept.
+ * faithful != 0: the pool choice as the reference makes it (threshold read at want - 1 after
+ * score_select fixed position want: it can take fewer than `want` pools, see
+ * orc_topk_quickselect).  faithful == 0: the pool choice by the contract (the `want` best by
+ * score, ties to the lower index), which is what the device path implements; the two agree
+ * whenever the reference's threshold is the smallest of its top set.  Returns the number of
+ * positions written to sel, or -1. */
+ORC_API int64_t orc_glm_select(const float *sc, int64_t n_comp, int64_t npos, int64_t kp, int64_t topk,
+                               int strict, int faithful, int32_t *sel) {
+    if (kp < 1) kp = 1;
+    const int64_t want = (topk + kp - 1) / kp;
+    if (want <= 0 || n_comp <= want) return -1;
+    int32_t *pools = malloc(sizeof(int32_t) * (size_t)want);
+    int64_t got;
+    if (faithful) {
+        got = orc_topk_quickselect(sc, n_comp, want, pools);
+    } else {
+        int32_t *asc = malloc(sizeof(int32_t) * (size_t)want);
+        const int64_t m = orc_topk_contract(sc, n_comp, want, asc);
+        float thr = INFINITY;
+        for (int64_t i = 0; i < m; i++) if (sc[asc[i]] < thr) thr = sc[asc[i]];
+        got = 0;
+        for (int pass = 0; pass < 2; pass++)
+            for (int64_t i = 0; i < m; i++) {
+                const float v = sc[asc[i]];
+                if (pass == 0 ? (v > thr) : (v == thr)) pools[got++] = asc[i];
+            }
+        free(asc);
+    }
+    int64_t n = 0;
+    for (int64_t i = 0; i < got; i++)
+        for (int64_t r = 0; r < kp; r++) sel[n++] = (int32_t)(pools[i] * kp + r);
+    free(pools);
+    const int64_t tail = npos % kp;
+    for (int64_t r = 0; r < tail; r++) sel[n++] = (int32_t)(npos - tail + r);
+    if (!strict && (n == 0 || sel[n - 1] != npos - 1)) sel[n++] = (int32_t)(npos - 1);
+    return n;
 }
 
 /* src/attention.c:486-525 (indexer_absorb once the pool has closed): one compressed indexer

@@ -381,6 +381,20 @@ def topk_quickselect(sc, want):
     return out[:got].copy()
 
 
+def glm_select(sc, npos, kpool, topk, strict=False, faithful=False):
+    """indexer_select after the scores (src/attention.c:585-620): the positions kept, or None for
+    "the whole prefix".  faithful: the pool choice exactly as the reference makes it; otherwise by
+    the contract (the device path)."""
+    sc = np.ascontiguousarray(sc, np.float32)
+    kp = max(int(kpool), 1)
+    want = (topk + kp - 1) // kp
+    sel = np.empty((want + 1) * kp + 1, np.int32)
+    lib().orc_glm_select.restype = C.c_int64
+    got = lib().orc_glm_select(_p(sc, C.c_float), C.c_int64(sc.size), C.c_int64(npos), C.c_int64(kp),
+                               C.c_int64(topk), int(bool(strict)), int(bool(faithful)), _p(sel, C.c_int32))
+    return None if got < 0 else sel[:got].copy()
+
+
 def ref_topk_scores(sc, k):
     """ds_topk_scores as compiled from the reference (src/ds_ops.c:310-338)."""
     R = ref()

@@ -1299,3 +1299,72 @@ def test_mm_select_host_operands(hip, orc):
         hip.mm_select(kv, n, iq, bs, keep, 4096)    # four heads per position: not an index-key cache
     idx.free()
     kv.free()
+
+
+# ------------------------------------------------------------------ the GLM selector behind the pool scores
+@pytest.mark.parametrize("n_comp,kp,topk,tail,strict,batch,kind", [
+    (5, 4, 8, 0, False, 1, "traced"),          # the hand-traced case: the query's position twice
+    (600, 4, 2048, 3, False, 3, "normal"),     # the GLM geometry (kpool 4, top-2048 -> 512 pools), a tail of three
+    (600, 4, 2048, 0, False, 3, "normal"),     # no tail: the self rule decides
+    (600, 4, 2048, 0, True, 2, "normal"),      # strict
+    (20000, 4, 2048, 1, False, 2, "normal"),   # the many-workgroup top-k under it
+    (3000, 1, 512, 0, False, 2, "ties"),       # kpool 1, ties at the threshold
+    (300, 4, 2048, 2, False, 2, "normal"),     # no more pools than wanted: the whole prefix
+    (5000, 8, 100, 5, False, 1, "last_high"),  # the last pool far above the threshold
+])
+def test_glm_select_on_device(hip, orc, n_comp, kp, topk, tail, strict, batch, kind):
+    """The rest of indexer_select (src/attention.c:585-620) on the device: pools by the contract,
+    the reference's list order, tail and self rule, against the oracle entry for entry; then the
+    list straight into the sparse MLA decode."""
+    import torch
+    say("[case] glm select", n_comp, kp, topk, tail, strict, batch, kind)
+    g = synth.rng(9100 + n_comp + tail)
+    npos = n_comp * kp + tail
+    want = (topk + kp - 1) // kp
+    max_sel = (want + 1) * kp + 7
+    if kind == "traced":
+        sc = np.array([[3, 1, 4, 1, 5]], np.float32)
+    elif kind == "ties":
+        sc = g.integers(0, 40, (batch, n_comp)).astype(np.float32)
+    else:
+        sc = g.standard_normal((batch, n_comp), dtype=np.float32)
+        if kind == "last_high":
+            sc[:, -1] = 50.0
+    d_sc = torch.from_numpy(sc).cuda()
+    d_sel = torch.full((batch, max_sel), 77, dtype=torch.int32, device="cuda")
+    d_n = torch.full((batch,), 77, dtype=torch.int32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    hip.glm_select_dev(d_sc, batch, n_comp, npos, kp, topk, strict, d_sel, max_sel, d_n, s)
+    torch.cuda.synchronize()
+    sel, ns = d_sel.cpu().numpy(), d_n.cpu().numpy()
+    for b in range(batch):
+        ref = orc.glm_select(sc[b], npos, kp, topk, strict=strict, faithful=False)
+        if ref is None:
+            assert ns[b] == -1 and list(sel[b, :npos]) == list(range(npos)) and (sel[b, npos:] == -1).all()
+            continue
+        assert ns[b] == ref.size, "query %d: %d positions, the oracle %d" % (b, ns[b], ref.size)
+        assert list(sel[b, :ref.size]) == list(ref), "query %d" % b
+        assert (sel[b, ref.size:] == -1).all()
+        if kind == "traced":
+            assert list(ref) == [16, 17, 18, 19, 8, 9, 10, 11, 19]
+        took = len(orc.topk_quickselect(sc[b], want))
+        if took == want:          # the reference's own threshold is the lowest of its top set: the same list
+            assert list(orc.glm_select(sc[b], npos, kp, topk, strict=strict, faithful=True)) == list(ref)
+    # the list as it stands into the sparse decode (a repeated position counts twice, as in the reference)
+    if npos >= 64:
+        c = synth.cfg3_mla_decode(npos, 128, seed=9200 + n_comp)
+        rows, scales = torch.from_numpy(c["rows"]).cuda(), torch.from_numpy(c["scales"]).cuda()
+        q = torch.from_numpy(np.repeat(c["q"][None], batch, 0).view(np.int16)).cuda()
+        out = torch.empty((batch, 128, synth.VDIM), dtype=torch.float32, device="cuda")
+        hip.mla_decode_dev(rows, scales, 0, 0, npos, batch, d_sel, max_sel, q, 128, c["scale"], out, s)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        for b in range(batch):
+            ref = orc.glm_select(sc[b], npos, kp, topk, strict=strict, faithful=False)
+            rsel = np.arange(npos, dtype=np.int32) if ref is None else ref
+            want_out = orc.mla_decode(c["q"], c["rows"], c["scales"], c["scale"], sel=rsel, nthreads=0)
+            assert_close(got[b], want_out, "glm select -> sparse decode, query %d" % b)
+    rc = hip.glm_select_dev(d_sc, batch, n_comp, npos + kp, kp, topk, strict, d_sel, max_sel, d_n, s, raw=True)
+    assert rc == 0 and "pools" in hip.last_error()
+    rc = hip.glm_select_dev(d_sc, batch, n_comp, npos, kp, topk, strict, d_sel, want * kp, d_n, s, raw=True)
+    assert rc == 0 and "max_sel" in hip.last_error()

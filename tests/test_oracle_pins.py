@@ -220,6 +220,59 @@ def test_topk_quickselect_hand_traced(orc, sc, want, traced):
     assert set(traced) <= set(int(i) for i in orc.topk_contract(sc, want))
 
 
+# The rest of indexer_select (src/attention.c:585-620) on the score vectors traced above, by hand:
+# pools -> positions c*kp + r in the reference's order (`> thr` ascending, then `== thr`), the tail
+# npos % kp, then npos - 1 unless it is the LAST entry already (:618 looks at sel[n-1] only, so a
+# selected last pool that is not the threshold pool is followed by a second copy of npos - 1).
+#   (sc, kp, topk, npos, strict) -> faithful list, contract-choice list (None: the same)
+GLM_SELECT_TRACED = [
+    # want 3; the reference takes pools 1, 3 only (under-selection), the contract 1, 3 then 4 (== thr 3)
+    ([1, 5, 2, 4, 3], 2, 6, 10, False, [2, 3, 6, 7, 9], [2, 3, 6, 7, 8, 9]),          # no tail; self pruned / self last already
+    ([1, 5, 2, 4, 3], 2, 6, 11, False, [2, 3, 6, 7, 10], [2, 3, 6, 7, 8, 9, 10]),      # tail of one position, which is the query
+    ([1, 5, 2, 4, 3], 2, 5, 10, True, [2, 3, 6, 7], [2, 3, 6, 7, 8, 9]),               # topk 5 -> want 3 as well; strict
+    # want 3; both take pools 0, 2 (> 3) then 1 (== 3)
+    ([5, 3, 4, 1, 2], 2, 5, 10, False, [0, 1, 4, 5, 2, 3, 9], None),                   # self pruned: appended
+    ([5, 3, 4, 1, 2], 2, 5, 10, True, [0, 1, 4, 5, 2, 3], None),
+    # want 2, kp 4: pool 4 (> 4) then pool 2 (== 4); the last pool is selected but not last in the list
+    ([3, 1, 4, 1, 5], 4, 8, 20, False, [16, 17, 18, 19, 8, 9, 10, 11, 19], None),      # the query twice
+    ([3, 1, 4, 1, 5], 4, 8, 22, False, [16, 17, 18, 19, 8, 9, 10, 11, 20, 21], None),  # tail of two, the query among them
+    ([3, 1, 4, 1, 5], 1, 2, 5, False, [4, 2, 4], None),                                # kp 1
+    ([3, 1, 4, 1, 5], 1, 2, 5, True, [4, 2], None),
+]
+
+
+@pytest.mark.parametrize("sc,kp,topk,npos,strict,faithful,contract", GLM_SELECT_TRACED)
+def test_glm_select_hand_traced(orc, sc, kp, topk, npos, strict, faithful, contract):
+    sc = np.array(sc, np.float32)
+    assert list(orc.glm_select(sc, npos, kp, topk, strict=strict, faithful=True)) == faithful
+    assert list(orc.glm_select(sc, npos, kp, topk, strict=strict, faithful=False)) == (contract or faithful)
+
+
+def test_glm_select_whole_prefix_and_agreement(orc):
+    # no more pools than wanted: "the whole prefix" (src/attention.c:558-559)
+    assert orc.glm_select(np.array([1, 2], np.float32), 9, 4, 8) is None
+    assert orc.glm_select(np.array([1, 2, 3], np.float32), 6, 2, 6, faithful=True) is None
+    # tie-free scores: whenever the reference's threshold is the smallest of its top set the two
+    # pool choices give the same list, entry for entry
+    g = synth.rng(77)
+    same = 0
+    for _ in range(300):
+        n_comp, kp = int(g.integers(5, 60)), int(g.integers(1, 5))
+        topk = int(g.integers(1, (n_comp - 1) * kp))
+        npos = n_comp * kp + int(g.integers(0, kp))
+        sc = g.permutation(n_comp).astype(np.float32)
+        a = orc.glm_select(sc, npos, kp, topk, faithful=True)
+        b = orc.glm_select(sc, npos, kp, topk, faithful=False)
+        want = (topk + kp - 1) // kp
+        took = len(orc.topk_quickselect(sc, want))
+        if took == want:
+            assert list(a) == list(b)
+            same += 1
+        else:
+            assert set(a) <= set(b) | {npos - 1}
+    assert same > 50
+
+
 def brute_topk(sc, k):
     order = sorted(range(len(sc)), key=lambda i: (-float(sc[i]), i))
     return sorted(order[:min(k, len(sc))])
