@@ -73,3 +73,69 @@ def test_mla_decode_static_declines_what_does_not_fit(hip):
     assert r.returncode == 0, r.stderr[-2000:]
     line = [l for l in r.stdout.splitlines() if l.startswith("RC ")][0]
     assert line.startswith("RC 0 UNTOUCHED True") and "static scratch" in line, line
+
+
+_CHILD_FIRST = r"""
+import sys
+import numpy as np
+import torch
+sys.path.insert(0, sys.argv[1])
+from cwick_amd import hip, synth
+assert hip.ready(), hip.last_error()
+c = synth.cfg3_mla_decode(9000, 128, seed=2104)
+rows = torch.from_numpy(c["rows"]).cuda(); scales = torch.from_numpy(c["scales"]).cuda()
+q = torch.from_numpy(c["q"].view(np.int16)).cuda()
+out = torch.full((128, synth.VDIM), float("nan"), dtype=torch.float32, device="cuda")
+out2 = torch.full((128, synth.VDIM), float("nan"), dtype=torch.float32, device="cuda")
+ref = torch.empty_like(out)
+ref2 = torch.empty_like(out)
+s = torch.cuda.Stream()
+torch.cuda.synchronize()
+free0, _ = torch.cuda.mem_get_info()
+# the very first call of this process into the entry point, under capture, no warm-up of any kind
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g, stream=s):
+    rc = hip.mla_decode_static_dev(rows, scales, 0, 0, 9000, 1, None, 9000, q, 128, c["scale"], out, s.cuda_stream, raw=True)
+g.replay()
+torch.cuda.synchronize()
+free1, _ = torch.cuda.mem_get_info()
+# a second capture, of a smaller shape, and an eager call: the device's free memory must not move
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2, stream=s):
+    rc2 = hip.mla_decode_static_dev(rows, scales, 0, 0, 9000, 1, None, 3000, q, 128, c["scale"], out2, s.cuda_stream, raw=True)
+g2.replay()
+torch.cuda.synchronize()
+free2, _ = torch.cuda.mem_get_info()
+rc3 = hip.mla_decode_static_dev(rows, scales, 0, 0, 9000, 1, None, 9000, q, 128, c["scale"], out, None, raw=True)
+torch.cuda.synchronize()
+free3, _ = torch.cuda.mem_get_info()
+hip.mla_decode_dev(rows, scales, 0, 0, 9000, 1, None, 9000, q, 128, c["scale"], ref, None)
+hip.mla_decode_dev(rows, scales, 0, 0, 9000, 1, None, 3000, q, 128, c["scale"], ref2, None)
+torch.cuda.synchronize()
+print("RC", rc, rc2, rc3, "SAME", bool(torch.equal(out.view(torch.int32), ref.view(torch.int32))),
+      "SAME2", bool(torch.equal(out2.view(torch.int32), ref2.view(torch.int32))),
+      "FREE", free0 - free1, free1 - free2, free2 - free3, "ERR", hip.last_error())
+"""
+
+
+def test_mla_decode_static_first_call_under_capture_allocates_nothing(hip):
+    """In a fresh process the first call ever made to the entry point is captured into a graph with no
+    warm-up (its one-time set-up -- the kernels' LDS attribute, the address of the scratch symbol --
+    runs under the capture) and the replay equals the allocating entry point bit for bit.  The
+    runtime loads the device image of the source file that holds the kernels and the 16 MiB area
+    at that first launch (once per process: at most 32 MiB go from the device's free memory
+    there); from then on -- a second capture of another shape, an eager call -- the free memory
+    does not move."""
+    import os
+    import subprocess
+    import sys
+    print("[case] mla_decode_static_dev: first call of a process, under capture", flush=True)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", _CHILD_FIRST, root], capture_output=True, text=True, timeout=150)
+    assert r.returncode == 0, r.stderr[-3000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("RC ")][0]
+    f = line.split()
+    assert f[1:4] == ["1", "1", "1"], line
+    assert "SAME True SAME2 True" in line, line
+    d = [int(x) for x in f[f.index("FREE") + 1:f.index("FREE") + 4]]
+    assert 0 <= d[0] <= 32 << 20 and d[1] == 0 and d[2] == 0, line
