@@ -53,8 +53,8 @@ constexpr int HW = 64;                        // heads per workgroup
 constexpr int NHQ = HW / 16;                  // 16-head blocks = scoring waves
 constexpr int NST = 3;                        // tile stages
 constexpr int NCOL = KDIM / 16;               // 36 sixteen-byte columns per row
-constexpr float LAZY = 4.0f;                  // the reference moves when a tile exceeds it by 2^LAZY
-constexpr int WEXP = 10;                      // fp16 weights are p * scale * 2^(WEXP - e), scale < 2^e
+constexpr float LAZY = 10.0f;                 // the reference moves when a tile exceeds it by 2^LAZY (fp16 probabilities up to 2^10)
+constexpr int WEXP = 4;                       // fp16 weights are p * scale * 2^(WEXP - e), scale < 2^e: below 2^(LAZY + WEXP) = 2^14
 constexpr int E_NONE = -1000;                 // no scale seen yet
 
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
@@ -140,6 +140,27 @@ constexpr uint32_t X_OFF = NST * TILE_B;                          // Smem::x
 constexpr uint32_t XCH_B = sizeof(Xch);
 constexpr uint32_t XC_OFF = NHQ * 2 * 4 * 16 * 4 * 4;             // Xch::c
 constexpr uint32_t XF_OFF = XC_OFF + NHQ * 16 * 4;                // Xch::moved
+
+// d = x * r[place n of the row]  /  d += x * r[place n of the row]: the factor comes out of one
+// lane of each row of sixteen (DPP row broadcast inside the multiply), so a row's sixteen factors
+// live in one register.  Assembly: the compiler folds a DPP move into a multiply but not into a
+// multiply-add.  It does not space an assembly statement from an MFMA whose result the statement
+// reads: x must have been written at least eleven instructions earlier (an 8-pass MFMA), which
+// the callers arrange by the order of their (volatile) statements.
+__device__ __forceinline__ void scaled_by_row_lane(float &d, float r, float x, int nsel, bool first) {
+#define CWICK_SBL_CASE(n)                                                                                         \
+    case n:                                                                                                       \
+        if (first) asm volatile("v_mul_f32_dpp %0, %1, %2 row_newbcast:" #n " row_mask:0xf bank_mask:0xf" : "=v"(d) : "v"(r), "v"(x)); \
+        else asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #n " row_mask:0xf bank_mask:0xf" : "+v"(d) : "v"(r), "v"(x));      \
+        break;
+    switch (nsel) {
+        CWICK_SBL_CASE(0) CWICK_SBL_CASE(1) CWICK_SBL_CASE(2) CWICK_SBL_CASE(3) CWICK_SBL_CASE(4) CWICK_SBL_CASE(5)
+        CWICK_SBL_CASE(6) CWICK_SBL_CASE(7) CWICK_SBL_CASE(8) CWICK_SBL_CASE(9) CWICK_SBL_CASE(10) CWICK_SBL_CASE(11)
+        CWICK_SBL_CASE(12) CWICK_SBL_CASE(13) CWICK_SBL_CASE(14) CWICK_SBL_CASE(15)
+        default: break;
+    }
+#undef CWICK_SBL_CASE
+}
 
 __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -322,7 +343,12 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
         // the next), the rope block's (columns 32 + 2 (g & 1)), this lane's four keys' scales
         const uint32_t k_off = (uint32_t)((2 * g) * (TK * 16) + n * 16);
         const uint32_t kr_off = (uint32_t)((32 + 2 * (g & 1)) * (TK * 16) + n * 16);
-        const uint32_t s_off = SC_OFF + (uint32_t)((4 * g) * 4);
+        // the scales of the tile's keys: lane (row g, place j) holds the scale of key
+        // 16 (j / 4) + 4 g + j % 4, the key that accumulator register j % 4 of key block j / 4 holds in
+        // this row: one register per dim block covers the tile (five 4-byte reads instead of twenty
+        // 16-byte ones, a quarter of what the four scoring waves read from LDS per tile), and the
+        // combination of the block products takes its factor from place 4 kb + i of the row
+        const uint32_t sr_off = SC_OFF + (uint32_t)((16 * (n >> 2) + 4 * g + (n & 3)) * 4);
         // where this lane's four probabilities of key block kb go: keys 16 (kb & 1) + 4 g + i of half kb >> 1
         const uint32_t xp_off = (uint32_t)(((hq * 2 * 4 + (g >> 1)) * 16 + n) * 16 + 2 * (g & 1) * 4);
         const uint32_t xc_off = XC_OFF + (uint32_t)((hq * 16 + n) * 4);
@@ -336,49 +362,66 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
                 // ---- scores S^T[key][head] for all 64 keys, heads 16 hq.. of tile t+1 ----
                 const uint32_t tb = st_sc;
                 const uint32_t xn = lds0 + X_OFF + (uint32_t)((t + 1) & 1) * XCH_B;
-                const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
                 f32x4 S[4];
+                float rsc[NBLK];
 #pragma unroll
-                for (int kb = 0; kb < 4; kb++) {
-                    const uint32_t ka = tb + k_off + (uint32_t)kb * 256u, kr = tb + kr_off + (uint32_t)kb * 256u;
-                    const uint32_t sa = tb + s_off + (uint32_t)kb * 64u;
-                    auto kfrag = [&](int b) -> i32x8 {
-                        const uint32_t a = b < 4 ? ka + (uint32_t)(8 * b) * (TK * 16) : kr;
-                        const u32x4 k0 = LDS_AT(lds_u32x4, a);
-                        const u32x4 k1 = LDS_AT(lds_u32x4, a + TK * 16);
-                        return (i32x8){(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
-                    };
-                    i32x8 kA = kfrag(0);
+                for (int b = 0; b < NBLK; b++) rsc[b] = LDS_AT(lds_f32, tb + sr_off + (uint32_t)b * (TK * 4));
+                // Fragment j = 5 kb + b (b = 4: the rope block).  Its MFMAs (hi and lo term, or the one
+                // rope instruction) are issued from assembly in a fixed order, its block product is
+                // folded into S three fragments later: between an MFMA and the statement that reads its
+                // result lie the MFMAs and folds of three other fragments (fifteen instructions or
+                // more, where an 8-pass MFMA asks for eleven), and a lo term accumulates into the
+                // registers its hi term wrote.
+                const uint32_t kbase = tb + k_off, krbase = tb + kr_off;
+                auto kfrag = [&](int j) -> i32x8 {
+                    const int kb = j / 5, b = j % 5;
+                    const uint32_t a = (b < 4 ? kbase + (uint32_t)(8 * b) * (TK * 16) : krbase) + (uint32_t)kb * 256u;
+                    const u32x4 k0 = LDS_AT(lds_u32x4, a);
+                    const u32x4 k1 = LDS_AT(lds_u32x4, a + TK * 16);
+                    return (i32x8){(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
+                };
+                const int one_scales = 0x7F7F7F7F;
+#define CWICK_P64_PAIR(A, K, QH, QL, SEL)                                                                         \
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %4, %5 " SEL "\n\t"                             \
+                 "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %3, %0, %4, %5 " SEL                                    \
+                 : "=&v"(A) : "v"(K), "v"(QH), "v"(QL), "v"(one_scales), "v"(qsc0))
+                f32x4 acc[4];
+                i32x8 kfr[3];
+                kfr[0] = kfrag(0);
+                kfr[1] = kfrag(1);
 #pragma unroll
-                    for (int b = 0; b < 4; b++) {
-                        const i32x8 kN = kfrag(b + 1);
-                        const f32x4 scb = LDS_AT(lds_f32x4, sa + (uint32_t)b * (TK * 4));
-                        f32x4 acc;
-                        if (b == 0) {
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 0, qsc0);
-                        } else if (b == 1) {
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 1, qsc0);
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 1, qsc0);
-                        } else if (b == 2) {
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 2, qsc0);
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 2, qsc0);
-                        } else {
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qhi[b], z4, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
-                            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qlo[b], acc, 0, 0, 0, 0x7F7F7F7F, 3, qsc0);
+                for (int j = 0; j < 23; j++) {
+                    if (j < 20) {
+                        const int b = j % 5;
+                        if (j + 2 < 20) kfr[(j + 2) % 3] = kfrag(j + 2);
+                        switch (b) {
+                            case 0: CWICK_P64_PAIR(acc[j % 4], kfr[j % 3], qhi[0], qlo[0], "op_sel:[0,0,0] op_sel_hi:[0,0,0]"); break;
+                            case 1: CWICK_P64_PAIR(acc[j % 4], kfr[j % 3], qhi[1], qlo[1], "op_sel:[0,1,0] op_sel_hi:[0,0,0]"); break;
+                            case 2: CWICK_P64_PAIR(acc[j % 4], kfr[j % 3], qhi[2], qlo[2], "op_sel:[0,0,0] op_sel_hi:[0,1,0]"); break;
+                            case 3: CWICK_P64_PAIR(acc[j % 4], kfr[j % 3], qhi[3], qlo[3], "op_sel:[0,1,0] op_sel_hi:[0,1,0]"); break;
+                            default:
+                                asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[0,0,0] op_sel_hi:[0,0,0]"
+                                             : "=&v"(acc[j % 4]) : "v"(kfr[j % 3]), "v"(qrope), "v"(one_scales), "v"(qsc1));
+                                break;
                         }
-                        if (b == 0) S[kb] = acc * scb;
-                        else S[kb] += acc * scb;
-                        kA = kN;
+                    } else {
+                        asm volatile("s_nop 3" ::: "memory");          // the last three folds have no MFMAs behind them
                     }
-                    {
-                        const f32x4 scb = LDS_AT(lds_f32x4, sa + 4u * (TK * 4));
-                        const f32x4 acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(kA, qrope, z4, 0, 0, 0, 0x7F7F7F7F, 0, qsc1);
-                        S[kb] += acc * scb;
+                    if (j >= 3) {
+                        const int f = j - 3, kb = f / 5, b = f % 5;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            float d = S[kb][i];
+                            scaled_by_row_lane(d, rsc[b], acc[f % 4][i], 4 * kb + i, b == 0);
+                            S[kb][i] = d;
+                        }
                     }
                 }
-                // positions past the query's last key (only in its last tile)
+#undef CWICK_P64_PAIR
+                // positions past the query's last key (only in its last tile; the empty statement keeps
+                // this a branch: as sixteen selects it would run in every step)
                 if (t + 1 == tail_tile && tail_keys < TK) {
+                    asm volatile("" ::: "memory");
 #pragma unroll
                     for (int kb = 0; kb < 4; kb++)
 #pragma unroll
