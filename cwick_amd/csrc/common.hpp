@@ -243,6 +243,11 @@ __device__ __forceinline__ uint32_t e4m3x2_to_bf16x2(uint32_t w) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// what place N of this lane's row of sixteen lanes holds (DPP row broadcast)
+template <int N>
+__device__ __forceinline__ uint32_t row_place(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + N, 0xF, 0xF, true);
+}
 // Lane l meets lane l ^ 16 (l ^ 32) without a trip through LDS: the rows of sixteen lanes (the
 // halves of the wave) trade places between two copies of the value, and a commutative
 // operation on the two copies is what a butterfly step would give, bit for bit.

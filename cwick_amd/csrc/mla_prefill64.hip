@@ -163,12 +163,6 @@ __device__ __forceinline__ void scaled_by_row_lane(float &d, float r, float x, i
 #undef CWICK_SBL_CASE
 }
 
-// what place N of this lane's row of sixteen holds (DPP row broadcast)
-template <int N>
-__device__ __forceinline__ uint32_t row_place(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + N, 0xF, 0xF, true);
-}
-
 __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     Smem &sm = *reinterpret_cast<Smem *>(smem_raw);

@@ -188,6 +188,7 @@ __device__ __forceinline__ uint32_t umax3(uint32_t a, uint32_t b, uint32_t c) {
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+typedef __attribute__((address_space(3))) f32x2 lds_f32x2;
 typedef __attribute__((address_space(3))) float lds_f32;
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
 // LDS is addressed by byte offsets held in ordinary integers (a generic pointer into LDS costs a
@@ -592,8 +593,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         // transpose-read addressing for V^T: lane i of 16-lane group g supplies key 8 g + (i >> 1),
         // bytes 8 (i & 1) .. +7 of the sixteen-byte column
         const uint32_t tr_off = (uint32_t)((8 * cw) * (TK * 16) + (8 * g + (n >> 1)) * 16 + 8 * (n & 1));
-        // scales of this wave's block for the keys of this lane's contraction slots (8 g .. +7 of each half)
-        const uint32_t sv_off = SC_OFF + (uint32_t)(cw * (TK * 4) + (8 * g) * 4);
+        // the two scales this lane turns into a pair of factors (see the loop)
+        const uint32_t sv_off = SC_OFF + (uint32_t)(cw * (TK * 4) + (32 * ((n & 7) >> 2) + 8 * g + 2 * (n & 3)) * 4);
         // the probabilities of this lane's slots: [head half][key half][g][n][4 dwords]
         const uint32_t pw_off = (uint32_t)((g * 16 + n) * 16);
         const uint32_t xml_off = XM_OFF + (uint32_t)(n * 16);
@@ -610,11 +611,11 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 // ---- values O^T[dim][head] += V^T W^T for dims 128 cw.., all 32 heads, tile t ----
                 const uint32_t tb = lds0 + (uint32_t)(t & (NST - 1)) * TILE_B;
                 const uint32_t xb = lds0 + X_OFF + (uint32_t)(t & 1) * XCH_B;
-                f32x4 sv[2][2];
-#pragma unroll
-                for (int kh = 0; kh < 2; kh++)
-#pragma unroll
-                    for (int q = 0; q < 2; q++) sv[kh][q] = LDS_AT(lds_f32x4, tb + sv_off + (uint32_t)(kh * 128 + q * 16));
+                // The sixteen lanes of a row share their contraction slots (keys 8 g .. 8 g + 7 of each
+                // half), so a row needs eight fp16 pairs of scale factors per tile: lane (g, n) reads
+                // the two scales of pair n & 7 (half (n & 7) >> 2, keys 8 g + 2 (n & 3) and the next),
+                // forms that one pair, and every lane takes the eight pairs out of the row by DPP.
+                const f32x2 sv = LDS_AT(lds_f32x2, tb + sv_off);
                 u32x4 pw[2][2];                           // [head half][key half]
 #pragma unroll
                 for (int h2 = 0; h2 < 2; h2++)
@@ -626,17 +627,8 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                 // they are positive, and a negative or NaN scale has the larger bit pattern too.
                 float ecorr = 1.0f;
                 {
-                    uint32_t sb[16];
-#pragma unroll
-                    for (int kh = 0; kh < 2; kh++)
-#pragma unroll
-                        for (int q = 0; q < 2; q++)
-#pragma unroll
-                            for (int i = 0; i < 4; i++) sb[(kh * 2 + q) * 4 + i] = __builtin_bit_cast(uint32_t, sv[kh][q][i]) & 0x7FFFFFFFu;
-                    uint32_t smax = umax3(sb[0], sb[1], sb[2]);
-#pragma unroll
-                    for (int i = 3; i < 15; i += 2) smax = umax3(smax, sb[i], sb[i + 1]);
-                    smax = smax > sb[15] ? smax : sb[15];
+                    const uint32_t b0 = __builtin_bit_cast(uint32_t, sv[0]) & 0x7FFFFFFFu, b1 = __builtin_bit_cast(uint32_t, sv[1]) & 0x7FFFFFFFu;
+                    const uint32_t smax = b0 > b1 ? b0 : b1;
                     if (__any(smax >= thr_bits && smax != 0u)) {
                         float sm_f = __builtin_bit_cast(float, smax);
                         sm_f = wave_max(sm_f);
@@ -649,14 +641,16 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
                         }
                     }
                 }
+                const uint32_t my_pair = pack_f16_rne(sv[0] * wfac, sv[1] * wfac);
                 u32x4 sw[2];                              // scale * 2^(WEXP - e_run) of the slots' keys, fp16 pairs
-#pragma unroll
-                for (int kh = 0; kh < 2; kh++) {
-                    sw[kh][0] = pack_f16_rne(sv[kh][0][0] * wfac, sv[kh][0][1] * wfac);
-                    sw[kh][1] = pack_f16_rne(sv[kh][0][2] * wfac, sv[kh][0][3] * wfac);
-                    sw[kh][2] = pack_f16_rne(sv[kh][1][0] * wfac, sv[kh][1][1] * wfac);
-                    sw[kh][3] = pack_f16_rne(sv[kh][1][2] * wfac, sv[kh][1][3] * wfac);
-                }
+                sw[0][0] = row_place<0>(my_pair);
+                sw[0][1] = row_place<1>(my_pair);
+                sw[0][2] = row_place<2>(my_pair);
+                sw[0][3] = row_place<3>(my_pair);
+                sw[1][0] = row_place<4>(my_pair);
+                sw[1][1] = row_place<5>(my_pair);
+                sw[1][2] = row_place<6>(my_pair);
+                sw[1][3] = row_place<7>(my_pair);
                 const uint32_t any_moved = (f0[0] | f0[1] | f0[2] | f0[3]) | (f1[0] | f1[1] | f1[2] | f1[3]);
                 if (__builtin_amdgcn_readfirstlane(any_moved) != 0u || ecorr != 1.0f) {
                     // a scoring wave left the common reference in this tile (or the weights'
