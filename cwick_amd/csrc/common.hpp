@@ -222,6 +222,15 @@ __device__ __forceinline__ uint32_t pack_f16_rne(float lo, float hi) {
     typedef __attribute__((ext_vector_type(2))) _Float16 v2h;
     return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f){lo, hi}, v2h));
 }
+// acc + both halves of a dword of two bf16 / two fp16, in fp32 (one dot-product instruction)
+__device__ __forceinline__ float pair_sum_bf16(uint32_t w, float acc) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 v2b;
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2b, w), __builtin_bit_cast(v2b, 0x3F803F80u), acc, false);
+}
+__device__ __forceinline__ float pair_sum_f16(uint32_t w, float acc) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2h;
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w), __builtin_bit_cast(v2h, 0x3C003C00u), acc, false);
+}
 // Two E4M3 bytes -> one dword of two fp16 (exact: E4M3 fits fp16's normal range)
 template <bool HI>
 __device__ __forceinline__ uint32_t e4m3x2_to_f16x2(uint32_t w) {

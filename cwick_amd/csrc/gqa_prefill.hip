@@ -293,7 +293,7 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                     pl[ks2][h] = pack_bf16_rne(s[8 * ks2 + 2 * h] - bf16lo_to_f32(pw[ks2][h]),
                                                s[8 * ks2 + 2 * h + 1] - bf16hi_to_f32(pw[ks2][h]));
                 else
-                    psum += bf16lo_to_f32(pw[ks2][h]) + bf16hi_to_f32(pw[ks2][h]);
+                    psum = pair_sum_bf16(pw[ks2][h], psum);
             }
         l_part[c] += psum;
     };
@@ -463,7 +463,9 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
         };
         // the running sums as opaque instructions: left to the compiler, the thirty-two additions
         // of a step sink to its end, a dependent chain behind the last MFMA
-        auto psum_add = [&](float &acc, float x) { asm volatile("v_add_f32 %0, %1, %0" : "+v"(acc) : "v"(x)); };
+        // (one dot-product instruction per packed pair: acc += lo * 1 + hi * 1)
+        const uint32_t ones_bf16 = 0x3F803F80u;
+        auto psum_pair = [&](float &acc, uint32_t w) { asm volatile("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(acc) : "s"(ones_bf16), "v"(w)); };
         auto pstep = [&](int t, int t3, f32x16 (&sc)[2], f32x16 (&sn)[2], const u32x4 (&pc)[2][2],
                          u32x4 (&pn)[2][2], float (&ps)[2]) {
             const int t3n = next3(t3);
@@ -507,10 +509,8 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
                     const uint32_t w1 = pack_bf16_rne(sc[1][i - 1], sc[1][i]);
                     pn[0][ks2][(i & 7) >> 1] = w0;
                     pn[1][ks2][(i & 7) >> 1] = w1;
-                    psum_add(p0, bf16lo_to_f32(w0));
-                    psum_add(p1, bf16lo_to_f32(w1));
-                    psum_add(p0, bf16hi_to_f32(w0));
-                    psum_add(p1, bf16hi_to_f32(w1));
+                    psum_pair(p0, w0);
+                    psum_pair(p1, w1);
                 }
                 if (!(i & 1)) {
                     if (i < 8) copy_one(src_k, dst_k, i >> 1);
