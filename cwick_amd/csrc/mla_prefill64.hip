@@ -36,7 +36,8 @@
 //   MFMAs and K reads 22.4, without the K reads alone 27.3: the two roles weigh the same and
 //   mostly add up; the matrix pipe is busy 2 176 of about 4 200 cycles per step and SIMD.
 //   Every K fragment is read from LDS by all four scoring waves (160 KB per tile); a timing build
-//   that read half of them ran 11 % faster.  A scoring wave of 32 heads x 32 keys would read each
+//   that read half of them ran 11 % faster (3 % since the scales are registers).  A scoring wave
+//   of 32 heads x 32 keys would read each
 //   fragment twice instead of four times, but its Q operands alone are 144 registers: with the
 //   loop's other values that does not fit the 256 of a wave (built: 24 of them reloaded from
 //   scratch every step), and Q fragments re-read from LDS give back what the K reads saved.
