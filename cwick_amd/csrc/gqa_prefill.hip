@@ -121,10 +121,17 @@ gqa_prefill_body(unsigned char *smem_raw, const uint16_t *__restrict__ K, const 
         row = row < last_key ? row : last_key;                  // masked anyway
         return base + (uint64_t)row * kv_stride32 + 64 * wave;
     };
+    // The 32 i bytes to the lane's source are the instruction's immediate offset (no address
+    // arithmetic per copy); the hardware adds that offset to the LDS address as well, so M0 is
+    // set 32 i bytes below the block.
     auto copy_one = [&](const uint16_t *src, uint32_t lds_tile, int i) {      // block 4 wave + i
-        const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK));
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     ::"v"(src + 16 * i), "s"(off) : "memory");
+        const uint32_t off = __builtin_amdgcn_readfirstlane(lds_tile + (uint32_t)((4 * wave + i) * PF_BLK - 32 * i));
+        switch (i) {
+            case 0: asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(off) : "memory"); break;
+            case 1: asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:32" ::"v"(src), "s"(off) : "memory"); break;
+            case 2: asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:64" ::"v"(src), "s"(off) : "memory"); break;
+            default: asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:96" ::"v"(src), "s"(off) : "memory"); break;
+        }
     };
     auto issue = [&](const uint16_t *base, uint32_t lds_tile, int tile) {
         const uint16_t *src = copy_src(base, tile);
