@@ -240,8 +240,14 @@ __global__ void __launch_bounds__(THREADS) mla_prefill64_kernel(const WideParams
         const uint64_t sp = live ? (uint64_t)(uintptr_t)scales + (uint64_t)(uint32_t)r * (NBLK * 4) : zsc;
         const uint32_t col_off = tile_off + (uint32_t)cw * (TK * 16);
         const uint64_t col_src = rp + 16 * cw;
-#pragma unroll
-        for (int k = 0; k < 9; k++) dma16(col_src + 64 * k, col_off + (uint32_t)(4 * k) * (TK * 16));
+        // the 64 k bytes to the lane's source are the instruction's immediate offset, which the
+        // hardware also adds to the LDS address: M0 is set that much below the column
+#define CWICK_P64_COL(k)                                                                                  \
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:" #k "*64"          \
+                 ::"v"(col_src), "s"(col_off + (uint32_t)(4 * k) * (TK * 16) - 64u * k) : "memory")
+        CWICK_P64_COL(0); CWICK_P64_COL(1); CWICK_P64_COL(2); CWICK_P64_COL(3); CWICK_P64_COL(4);
+        CWICK_P64_COL(5); CWICK_P64_COL(6); CWICK_P64_COL(7); CWICK_P64_COL(8);
+#undef CWICK_P64_COL
         dma4(sp + 4 * cw, tile_off + SC_OFF + (uint32_t)cw * (TK * 4));
         if (cw == 0) dma4(sp + 16, tile_off + SC_OFF + 4u * (TK * 4));
     };
