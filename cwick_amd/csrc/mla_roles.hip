@@ -298,9 +298,13 @@ __global__ void __launch_bounds__(THREADS) mla_roles_kernel(const Params p) {
         // columns wave, wave + 12, wave + 24 (all below 36) and, for the first five waves, scale block `wave`
         const uint32_t col_off = tile_off + (uint32_t)wave * (TK * 16);
         const uint64_t col_src = rp + 16 * wave;
+        // (the 192 and 384 bytes to the lane's source are the instruction's immediate offset, which
+        // the hardware also adds to the LDS address: M0 is set that much below the column)
         dma16(col_src, col_off);
-        dma16(col_src + 192, col_off + 12 * (TK * 16));
-        dma16(col_src + 384, col_off + 24 * (TK * 16));
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:192"
+                     ::"v"(col_src), "s"(col_off + 12 * (TK * 16) - 192u) : "memory");
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:384"
+                     ::"v"(col_src), "s"(col_off + 24 * (TK * 16) - 384u) : "memory");
         if (wave < NBLK) dma4(sp + 4 * wave, tile_off + SC_OFF + (uint32_t)wave * (TK * 4));
         if (SEL && wave == 0) mark(r, tile_off);
     };
