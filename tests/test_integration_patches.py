@@ -1,4 +1,4 @@
-"""The guards of INTEGRATION.md as patches against the engine's own files (integration/*.patch:
+"""The backend's guards as patches against the engine's own files (integration/*.patch:
 added lines only): each applies to a copy of the reference file it names and the patched file
 compiles as C11 against the engine's headers and include/cwick_hip.h, with the backend compiled in
 (-DCWICK_WITH_HIP) and without it.  No link step: the engine cannot be linked here.  Runs only
