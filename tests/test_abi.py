@@ -4,6 +4,7 @@ import ctypes
 import os
 import re
 import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -63,3 +64,12 @@ def test_declines_without_a_gpu():
     assert L.cwick_hip_kv_create(16, 4, 256) is None
     assert L.cwick_hip_force(0) == 0 and L.cwick_hip_ready() == 0
     assert "not selected" in hip.last_error() or "unavailable" in hip.last_error()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py shows one GPU's share of the path: --gpus N with N above 1 ends with a message
+    that says so, before anything touches a device."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "--gpus 2 is not run" in r.stderr + r.stdout
+    assert not r.stdout.strip().startswith("{")
